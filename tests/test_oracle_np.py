@@ -1,0 +1,256 @@
+"""Pins the numpy oracle: exact rational closed forms on the reference's own arange fixtures
+(MeshFlowCPU.ipynb cells 2-4), brute-force index enumeration, partition invariants, and the
+identity sliced == unsliced == dense that the reference itself asserts (ipynb:80,102,111,130-132;
+TensorParallel.py:447,452,457)."""
+import itertools
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import meshslice_oracle as orc
+
+
+# ---------------------------------------------------------------- slice selector
+def _sel_bruteforce(L, S, B, k):
+    """Enumerate the (L/(S*B), S, B) view element by element, keep axis-1 index k."""
+    out = []
+    g = 0
+    for q in range(L // (S * B)):
+        for s in range(S):
+            for b in range(B):
+                if s == k:
+                    out.append(g)
+                g += 1
+    return out
+
+
+@pytest.mark.parametrize("L,S,B", [(16, 2, 2), (64, 4, 8), (64, 8, 8), (96, 3, 8), (48, 1, 8), (120, 5, 4)])
+def test_sel_matches_reshape_enumeration(L, S, B):
+    seen = []
+    for k in range(S):
+        s = orc.sel(L, S, B, k)
+        assert list(s) == _sel_bruteforce(L, S, B, k)
+        assert len(s) == L // S
+        seen.extend(s)
+    assert sorted(seen) == list(range(L))          # slices partition the range
+
+
+def test_sel_rejects_bad_shapes():
+    with pytest.raises(ValueError):
+        orc.sel(60, 4, 8, 0)
+    with pytest.raises(ValueError):
+        orc.sel(64, 4, 8, 4)
+
+
+# ---------------------------------------------------------------- bf16 rounding
+def test_bf16_round_matches_torch_and_special_values():
+    rng = np.random.default_rng(1)
+    x = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32),
+        (rng.standard_normal(2000) * 1e-40).astype(np.float32),          # subnormals
+        np.array([0.0, -0.0, np.inf, -np.inf, 1.0, 1.00390625, 1.01171875,  # ties: 1+2^-8, 1+3*2^-8
+                  3.3895314e38, 65504.0, 1e-45], np.float32),
+    ])
+    want = torch.from_numpy(x).to(torch.bfloat16).to(torch.float32).numpy()
+    got = orc.bf16_round(x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert orc.bf16_round(np.float32([1.00390625]))[0] == 1.0            # tie -> even (down)
+    assert orc.bf16_round(np.float32([1.01171875]))[0] == 1.015625       # tie -> even (up)
+    assert np.isnan(orc.bf16_round(np.float32([np.nan]))[0])
+    assert np.array_equal(orc.bits_to_f32(orc.bf16_bits(x)).view(np.uint32), got.view(np.uint32))
+
+
+# ---------------------------------------------------------------- notebook fixture, exact
+def _notebook_exact():
+    """Exact integer numerators of Y, dX, dW for the notebook inputs (all operands are
+    integers over a power of two, so every product and sum is exact)."""
+    Bt, I, O = 512, 256, 1024
+    r = np.arange(Bt, dtype=object)[:, None]
+    c = np.arange(O, dtype=object)[None, :]
+    s1 = I * (I - 1) // 2
+    s2 = (I - 1) * I * (2 * I - 1) // 6
+    # Y[r,c] = sum_k (r*I+k)*(k*O+c) / ((B*I)*(I*O))
+    Ynum = r * I * O * s1 + r * I * c * I + O * s2 + c * s1
+    Yden = (Bt * I) * (I * O)
+    # dX[r,i] = sum_o W[i,o] / (B*O) = sum_o (i*O+o) / ((I*O)*(B*O))
+    i = np.arange(I, dtype=object)[None, :]
+    dXnum = np.repeat(i * O * O + O * (O - 1) // 2, Bt, axis=0)
+    dXden = (I * O) * (Bt * O)
+    # dW[i,o] = sum_b X[b,i] / (B*O) = sum_b (b*I+i) / ((B*I)*(B*O))
+    ii = np.arange(I, dtype=object)[:, None]
+    dWnum = np.repeat(I * Bt * (Bt - 1) // 2 + Bt * ii, O, axis=1)
+    dWden = (Bt * I) * (Bt * O)
+    f = lambda num, den: (num.astype(np.float64) / float(den))
+    return f(Ynum, Yden), f(dXnum, dXden), f(dWnum, dWden)
+
+
+@pytest.fixture(scope="module")
+def nb():
+    d = orc.notebook_inputs(np.float64)
+    # arange / 2^k is exact in fp32, so the float64 copies carry the reference's fp32 values
+    assert np.array_equal(d["X"], orc.notebook_inputs(np.float32)["X"].astype(np.float64))
+    return d
+
+
+def test_notebook_dense_equals_exact_closed_form(nb):
+    Y, dX, dW = _notebook_exact()
+    assert np.array_equal(orc.dense("os", nb["X"], nb["W"]), Y)
+    assert np.array_equal(orc.dense("ls", nb["dY"], nb["W"]), dX)
+    assert np.array_equal(orc.dense("rs", nb["X"], nb["dY"]), dW)
+    # a spot value by exact rational arithmetic, independent of the polynomial above
+    r, c = 311, 777
+    v = sum(Fraction((r * 256 + k) * (k * 1024 + c), (512 * 256) * (256 * 1024)) for k in range(256))
+    assert Y[r, c] == float(v)
+
+
+@pytest.mark.parametrize("dataflow", ["os", "ls", "rs"])
+def test_notebook_collective_and_meshflow_equal_exact(nb, dataflow):
+    Y, dX, dW = _notebook_exact()
+    R, C = nb["mesh"]
+    X, W, want = {"os": (nb["X"], nb["W"], Y), "ls": (nb["dY"], nb["W"], dX), "rs": (nb["X"], nb["dY"], dW)}[dataflow]
+    got_c = orc.literal_collective(dataflow, X, W, R, C)
+    got_m = orc.literal_meshflow(dataflow, X, W, R, C, nb["K"], nb["blocksize"])
+    assert np.array_equal(got_c, want)
+    assert np.array_equal(got_m, want)            # exact: every partial sum is an integer / 2^k
+
+
+@pytest.mark.parametrize("dataflow", ["os", "ls", "rs"])
+def test_notebook_device_blocks_and_assembly(nb, dataflow):
+    Y, dX, dW = _notebook_exact()
+    R, C = nb["mesh"]; S = nb["K"]; B = nb["blocksize"]
+    X, W, want = {"os": (nb["X"], nb["W"], Y), "ls": (nb["dY"], nb["W"], dX), "rs": (nb["X"], nb["dY"], dW)}[dataflow]
+    orc.check_divisibility(dataflow, X.shape, W.shape, R, C, S, B)
+    if dataflow == "os":
+        for i, j in itertools.product(range(R), range(C)):
+            A, Bs = orc.device_operands_os(X, W, R, C, i, j, S, B)
+            assert A[0].shape == (512 // R, 256 // S) and Bs[0].shape == (256 // S, 1024 // C)
+            assert np.array_equal(orc.oracle_os_block(A, Bs), orc.shard(want, R, C, i, j))
+    elif dataflow == "ls":
+        for i in range(R):
+            chunks = []
+            for j in range(C):
+                A, Ws = orc.device_operands_ls(X, W, R, C, i, j, S, B)
+                chunks.append(orc.oracle_ls_chunks(A, Ws))
+            for j in range(C):
+                assert np.array_equal(orc.assemble_ls(chunks, R, C, j, S, B), orc.shard(want, R, C, i, j))
+    else:
+        for j in range(C):
+            chunks = []
+            for i in range(R):
+                Xs, Wl = orc.device_operands_rs(X, W, R, C, i, j, S, B)
+                chunks.append(orc.oracle_rs_chunks(Xs, Wl))
+            for i in range(R):
+                assert np.array_equal(orc.assemble_rs(chunks, R, C, i, S, B), orc.shard(want, R, C, i, j))
+
+
+# ---------------------------------------------------------------- integer-valued random cases, exact
+def _int_mats(rng, shape_x, shape_w):
+    return (rng.integers(-4, 5, size=shape_x).astype(np.float64),
+            rng.integers(-4, 5, size=shape_w).astype(np.float64))
+
+
+CASES = [  # (R, C, S, B, dims)  dims = (a, b, c): os X[a,b] W[b,c]; ls X[a,b] W[c,b]; rs X[a,b] W[a,c]
+    (2, 2, 2, 2, (16, 16, 16)),
+    (2, 2, 1, 2, (8, 8, 8)),
+    (4, 2, 4, 8, (64, 128, 128)),
+    (2, 4, 8, 8, (32, 256, 256)),
+    (1, 1, 4, 8, (8, 32, 64)),
+    (2, 2, 3, 4, (24, 48, 48)),
+]
+
+
+@pytest.mark.parametrize("R,C,S,B,dims", CASES)
+@pytest.mark.parametrize("dataflow", ["os", "ls", "rs"])
+def test_literal_meshflow_equals_dense_and_closed_form(R, C, S, B, dims, dataflow):
+    rng = np.random.default_rng(hash((R, C, S, B, dataflow)) % (1 << 31))
+    a, b, c = dims
+    if dataflow == "os":
+        X, W = _int_mats(rng, (a, b), (b, c))
+    elif dataflow == "ls":
+        X, W = _int_mats(rng, (a, b), (c, b))
+    else:
+        X, W = _int_mats(rng, (b, a * 4), (b, c))      # N = 4a keeps N % (S*B*R) == 0
+    try:
+        orc.check_divisibility(dataflow, X.shape, W.shape, R, C, S, B)
+    except ValueError:
+        pytest.skip("shape not admissible for this mesh/slice count")
+    want = orc.dense(dataflow, X, W)
+    assert np.array_equal(orc.literal_collective(dataflow, X, W, R, C), want)
+    if not (dataflow == "os" and S == 1):
+        assert np.array_equal(orc.literal_meshflow(dataflow, X, W, R, C, S, B), want)
+    # closed-form device operands + block oracle + mesh completion reproduce the same thing
+    if dataflow == "os":
+        for i, j in itertools.product(range(R), range(C)):
+            assert np.array_equal(orc.oracle_os_block(*orc.device_operands_os(X, W, R, C, i, j, S, B)),
+                                  orc.shard(want, R, C, i, j))
+    elif dataflow == "ls":
+        for i in range(R):
+            ch = [orc.oracle_ls_chunks(*orc.device_operands_ls(X, W, R, C, i, j, S, B)) for j in range(C)]
+            for j in range(C):
+                assert np.array_equal(orc.assemble_ls(ch, R, C, j, S, B), orc.shard(want, R, C, i, j))
+    else:
+        for j in range(C):
+            ch = [orc.oracle_rs_chunks(*orc.device_operands_rs(X, W, R, C, i, j, S, B)) for i in range(R)]
+            for i in range(R):
+                assert np.array_equal(orc.assemble_rs(ch, R, C, i, S, B), orc.shard(want, R, C, i, j))
+
+
+def test_meshflow_os_k1_quirk_is_a_double_count():
+    """TensorParallel.py:163 asks for slice 1 of a 1-slice view; dynamic_slice clamps it to slice 0
+    and :172 adds it again, so the reference's sliced OS body returns 2*X@W for K=1.  The build
+    never routes S=1 through that body (S=1 is the 'collective' contraction)."""
+    rng = np.random.default_rng(5)
+    X, W = _int_mats(rng, (8, 16), (16, 8))
+    got = orc.literal_meshflow_os(X, W, 2, 2, 1, 2)
+    assert np.array_equal(got, 2.0 * (X @ W))
+    assert np.array_equal(orc.literal_meshflow_os(X, W, 2, 2, 2, 2), X @ W)
+
+
+def test_selfcheck_fixture_chain_matches_polynomial():
+    """TensorParallel.py:433-457 chain Yo=OS(X,W), LS(Yo,W), RS(X,Yo) on the 4x4 mesh; checked on
+    one device block each against the dense product and a polynomial closed form of X@W."""
+    d = orc.selfcheck_inputs(np.float32)
+    X, W = d["X"].astype(np.float64), d["W"].astype(np.float64)
+    R, C = d["mesh"]; S, B = d["K"], d["blocksize"]
+    i, j = 2, 1
+    A, Bs = orc.device_operands_os(X, W, R, C, i, j, S, B)
+    blk = orc.oracle_os_block(A, Bs)
+    n, dd = X.shape[0], X.shape[1]
+    o = W.shape[1]
+    r = np.arange(i * n // R, (i + 1) * n // R, dtype=np.float64)[:, None]
+    c = np.arange(j * o // C, (j + 1) * o // C, dtype=np.float64)[None, :]
+    s1 = dd * (dd - 1) / 2
+    s2 = (dd - 1) * dd * (2 * dd - 1) / 6
+    poly = (r * dd * o * s1 + r * dd * c * dd + o * s2 + c * s1) / (float(n * dd) * float(4 * dd * dd))
+    assert orc.rel_frobenius(blk, poly) < 1e-6     # fp32 rounding of arange/denominator only
+    assert orc.rel_frobenius(blk, (X @ W)[orc.block_range(n, R, i), orc.block_range(o, C, j)]) < 1e-13
+
+
+# ---------------------------------------------------------------- backward wiring
+@pytest.mark.parametrize("dataflow", ["os", "ls", "rs"])
+def test_vjp_permutation_matches_autograd(dataflow):
+    """ShardedLayers.py:41-81: the (fwd, dx, dw) triples are (OS,LS,RS), (LS,OS,RS), (RS,LS,OS)."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(12, 20, dtype=torch.float64, generator=g, requires_grad=True)
+    if dataflow == "os":      # y = x @ w, w [in,out]
+        w = torch.randn(20, 28, dtype=torch.float64, generator=g, requires_grad=True)
+        y = x @ w
+    elif dataflow == "ls":    # y = x @ w^T, w [out,in]
+        w = torch.randn(28, 20, dtype=torch.float64, generator=g, requires_grad=True)
+        y = x @ w.t()
+    else:                     # y = x^T @ w, x [in, tokens]
+        w = torch.randn(12, 28, dtype=torch.float64, generator=g, requires_grad=True)
+        y = x.t() @ w
+    dy = torch.randn(*y.shape, dtype=torch.float64, generator=g)
+    y.backward(dy)
+    xn, wn, dyn = x.detach().numpy(), w.detach().numpy(), dy.numpy()
+    if dataflow == "os":
+        dx, dw = orc.dense("ls", dyn, wn), orc.dense("rs", xn, dyn)
+    elif dataflow == "ls":
+        dx, dw = orc.dense("os", dyn, wn), orc.dense("rs", dyn, xn)
+    else:
+        dx, dw = orc.dense("ls", wn, dyn), orc.dense("os", xn, dyn)
+    assert np.allclose(dx, x.grad.numpy(), rtol=1e-12, atol=1e-12)
+    assert np.allclose(dw, w.grad.numpy(), rtol=1e-12, atol=1e-12)
