@@ -1,0 +1,106 @@
+/* meshslice_hip.h — C ABI of libmeshslice_hip.so
+ *
+ * MI355X (gfx950) kernels for the per-device local contraction of MeshSlice's sliced 2-D GEMM.
+ * One call = the whole local work of ONE mesh device for ONE sharded matmul: all S slices that
+ * the device receives from its all-gathers (output-stationary), or all S partial-output chunks
+ * that it hands to its reduce-scatters (LHS- / RHS-stationary).
+ *
+ * The reference has no FFI seam; each entry point replaces the einsum / matmul calls of one
+ * per-device body of the reference's TensorParallel.py (cited per function).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller, 16-byte aligned; the slice / chunk
+ *     pointer arrays themselves are HOST arrays of S device pointers, read during the call;
+ *   - matrices are row-major with a leading dimension in ELEMENTS;
+ *   - in_dtype / out_dtype: MS_DTYPE_F32 or MS_DTYPE_BF16; products accumulate in fp32 across the
+ *     full contraction (all slices) and are rounded once (round-to-nearest-even) on output;
+ *   - contiguous extents and leading dimensions must be multiples of 8 (bf16) or 4 (fp32)
+ *     elements — implied by the reference's block size of 8; other extents are free;
+ *   - calls are asynchronous on `stream` (a hipStream_t; NULL = the default stream);
+ *   - return 0 on success, MS_ERR_* (< 0) otherwise; ms_last_error() then describes the failure;
+ *   - the library allocates no device memory and keeps no state besides a per-thread error text.
+ */
+#ifndef MESHSLICE_HIP_H
+#define MESHSLICE_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MS_DTYPE_F32 0
+#define MS_DTYPE_BF16 1
+
+#define MS_OK 0
+#define MS_ERR_ARG (-1)         /* bad argument: null pointer, size <= 0, alignment / divisibility */
+#define MS_ERR_UNSUPPORTED (-2) /* dtype combination or device architecture not supported */
+#define MS_ERR_HIP (-3)         /* a HIP runtime call failed */
+
+#define MS_MAX_SLICES 64        /* largest S accepted by one call */
+
+/* ms_query() selectors */
+#define MS_QUERY_CU_COUNT 0     /* compute units of the current device */
+#define MS_QUERY_CLOCK_KHZ 1    /* peak engine clock */
+#define MS_QUERY_IS_GFX950 2    /* 1 if the current device is gfx950 */
+#define MS_QUERY_LDS_BYTES 3    /* LDS bytes per workgroup */
+#define MS_QUERY_MAX_SLICES 4   /* MS_MAX_SLICES */
+
+/* Library version, major*10000 + minor*100 + patch. */
+int ms_version(void);
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char *ms_last_error(void);
+
+/* Device / library facts; returns -1 for an unknown selector or on a HIP error. */
+long ms_query(int what);
+
+/* Output-stationary: C[m,n] = sum_{s<S} A_s[m,k_slice] @ B_s[k_slice,n].
+ * Replaces the contractions of MeshFlow_OS (reference TensorParallel.py:162,167,172); with S == 1
+ * it is Collective_OS (TensorParallel.py:22).  A_s is the s-th all-gathered column slice of the
+ * activations (lda), B_s the s-th all-gathered row slice of the weights (ldb).  C is written in
+ * out_dtype (ldc). */
+int ms_gemm_os(const void *const *A_slices, const void *const *B_slices, int S,
+               int m, int n, int k_slice, int lda, int ldb,
+               void *C, int ldc, int in_dtype, int out_dtype, void *stream);
+
+/* LHS-stationary: for s < S, Y_s[m,n_slice] = A[m,k] @ W_s[n_slice,k]^T  (fp32 out).
+ * Replaces the contractions of MeshFlow_LS (TensorParallel.py:181,187); S == 1 is Collective_LS
+ * (TensorParallel.py:26).  A is the device's own shard; W_s the s-th all-gathered row slice of the
+ * [out,in] weights; Y_s is the partial-output chunk the mesh reduce-scatters over its columns.
+ * Chunks are produced in slice order: every tile of Y_s is scheduled before any tile of Y_{s+1}. */
+int ms_gemm_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S,
+               int m, int n_slice, int k,
+               float *const *Y_chunks, int ldy, int in_dtype, void *stream);
+
+/* RHS-stationary: for s < S, Y_s[m_slice,n] = X_s[k,m_slice]^T @ W[k,n]  (fp32 out).
+ * Replaces the contractions of MeshFlow_RS (TensorParallel.py:203,209); S == 1 is Collective_RS
+ * (TensorParallel.py:31).  X_s is the s-th all-gathered column slice of the [in,tokens] operand,
+ * stored [k,m_slice] and used transposed; W is the device's own shard. */
+int ms_gemm_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int S,
+               int m_slice, int n, int k,
+               float *const *Y_chunks, int ldy, int in_dtype, void *stream);
+
+/* Timing helpers (replace the wall-clock loop of CostModel.estimateMatmul, reference
+ * CostModel.py:74-98): run the same call `warmup` times untimed, then `reps` times, each launch
+ * bracketed by HIP events on `stream`; ms_out[r] receives the r-th launch's milliseconds.
+ * Synchronise the stream before returning. */
+int ms_time_os(const void *const *A_slices, const void *const *B_slices, int S,
+               int m, int n, int k_slice, int lda, int ldb,
+               void *C, int ldc, int in_dtype, int out_dtype, void *stream,
+               int warmup, int reps, float *ms_out);
+int ms_time_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S,
+               int m, int n_slice, int k,
+               float *const *Y_chunks, int ldy, int in_dtype, void *stream,
+               int warmup, int reps, float *ms_out);
+int ms_time_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int S,
+               int m_slice, int n, int k,
+               float *const *Y_chunks, int ldy, int in_dtype, void *stream,
+               int warmup, int reps, float *ms_out);
+
+/* Tuning knob for experiments: selects the bf16 kernel variant used by later calls on this
+ * thread (0 = library default).  Unknown ids are rejected with MS_ERR_ARG. */
+int ms_set_variant(int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MESHSLICE_HIP_H */

@@ -1,0 +1,99 @@
+"""ctypes binding of libmeshslice_hip.so (the C ABI declared in include/meshslice_hip.h).
+
+There is no CPU fallback: if the shared library has not been built, or a call fails, an exception is
+raised.  Build it with ``python -c "import __graft_entry__ as g; g.build()"`` or
+``make -C meshslice_amd/csrc``.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+MS_DTYPE_F32 = 0
+MS_DTYPE_BF16 = 1
+MS_OK = 0
+MS_ERR_ARG = -1
+MS_ERR_UNSUPPORTED = -2
+MS_ERR_HIP = -3
+MS_QUERY_CU_COUNT = 0
+MS_QUERY_CLOCK_KHZ = 1
+MS_QUERY_IS_GFX950 = 2
+MS_QUERY_LDS_BYTES = 3
+MS_QUERY_MAX_SLICES = 4
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmeshslice_hip.so")
+
+EXPORTS = (
+    "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
+    "ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs",
+    "ms_time_os", "ms_time_ls", "ms_time_rs",
+)
+
+_lock = threading.Lock()
+_lib = None
+
+
+class MeshSliceError(RuntimeError):
+    """A call into libmeshslice_hip.so failed (HIP error or unsupported configuration)."""
+
+
+def _declare(lib):
+    c_int, c_vp, c_long = ctypes.c_int, ctypes.c_void_p, ctypes.c_long
+    vpp = ctypes.POINTER(ctypes.c_void_p)
+    fp = ctypes.POINTER(ctypes.c_float)
+    lib.ms_version.argtypes = []
+    lib.ms_version.restype = c_int
+    lib.ms_last_error.argtypes = []
+    lib.ms_last_error.restype = ctypes.c_char_p
+    lib.ms_query.argtypes = [c_int]
+    lib.ms_query.restype = c_long
+    lib.ms_set_variant.argtypes = [c_int]
+    lib.ms_set_variant.restype = c_int
+    os_args = [vpp, vpp, c_int, c_int, c_int, c_int, c_int, c_int, c_vp, c_int, c_int, c_int, c_vp]
+    ls_args = [c_vp, c_int, vpp, c_int, c_int, c_int, c_int, c_int, vpp, c_int, c_int, c_vp]
+    rs_args = [vpp, c_int, c_vp, c_int, c_int, c_int, c_int, c_int, vpp, c_int, c_int, c_vp]
+    lib.ms_gemm_os.argtypes = os_args
+    lib.ms_gemm_ls.argtypes = ls_args
+    lib.ms_gemm_rs.argtypes = rs_args
+    lib.ms_time_os.argtypes = os_args + [c_int, c_int, fp]
+    lib.ms_time_ls.argtypes = ls_args + [c_int, c_int, fp]
+    lib.ms_time_rs.argtypes = rs_args + [c_int, c_int, fp]
+    for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_time_os", "ms_time_ls", "ms_time_rs"):
+        getattr(lib, n).restype = c_int
+
+
+def load():
+    """Return the loaded library; raise MeshSliceError if it has not been built."""
+    global _lib
+    with _lock:
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise MeshSliceError(
+                    f"{LIB_PATH} is missing: the HIP extension has not been built "
+                    "(run __graft_entry__.build() or `make -C meshslice_amd/csrc`); there is no CPU fallback")
+            lib = ctypes.CDLL(LIB_PATH)
+            _declare(lib)
+            _lib = lib
+        return _lib
+
+
+def last_error() -> str:
+    return load().ms_last_error().decode("utf-8", "replace")
+
+
+def check(rc: int) -> None:
+    """Map a C return code to the exception the reference's Python would raise in that situation:
+    shape/argument problems -> ValueError, everything else -> MeshSliceError."""
+    if rc == MS_OK:
+        return
+    msg = last_error()
+    if rc == MS_ERR_ARG:
+        raise ValueError(msg)
+    raise MeshSliceError(f"libmeshslice_hip error {rc}: {msg}")
+
+
+def ptr_array(ptrs):
+    arr = (ctypes.c_void_p * len(ptrs))(*[int(p) for p in ptrs])
+    return ctypes.cast(arr, ctypes.POINTER(ctypes.c_void_p)), arr

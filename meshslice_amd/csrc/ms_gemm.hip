@@ -1,0 +1,304 @@
+// libmeshslice_hip.so — C ABI over the gfx950 GEMM kernels (declarations: include/meshslice_hip.h).
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "meshslice_hip.h"
+
+#include "ms_gemm_bf16.hip.inc"
+#include "ms_gemm_f32.hip.inc"
+
+#define MS_API extern "C" __attribute__((visibility("default")))
+
+// Every kernel variant is instantiated explicitly: with implicit instantiation alone the host
+// compiler leaves some of the launch stubs undefined.
+#define MS_INSTANTIATE(BM, BN, WGM, WGN)                                                                  \
+  template __global__ void msk::gemm_bf16_kernel<BM, BN, WGM, WGN, true, false, true>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_kernel<BM, BN, WGM, WGN, true, false, false>(const msk::GemmArgs);  \
+  template __global__ void msk::gemm_bf16_kernel<BM, BN, WGM, WGN, true, true, false>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_kernel<BM, BN, WGM, WGN, false, false, false>(const msk::GemmArgs);
+MS_INSTANTIATE(256, 256, 2, 2)
+MS_INSTANTIATE(256, 256, 2, 4)
+MS_INSTANTIATE(128, 128, 2, 2)
+#undef MS_INSTANTIATE
+
+namespace {
+
+thread_local char g_err[512] = "";
+thread_local int g_variant = 0;
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+#define MS_HIP(call)                                                                        \
+  do {                                                                                      \
+    hipError_t e_ = (call);                                                                 \
+    if (e_ != hipSuccess) return fail(MS_ERR_HIP, "%s failed: %s", #call, hipGetErrorString(e_)); \
+  } while (0)
+
+struct DevInfo {
+  int valid, cus, clock_khz, gfx950, lds;
+};
+DevInfo g_dev[64];
+
+int dev_info(DevInfo **out) {
+  int d = 0;
+  MS_HIP(hipGetDevice(&d));
+  if (d < 0 || d >= 64) return fail(MS_ERR_HIP, "device ordinal %d out of range", d);
+  if (!__atomic_load_n(&g_dev[d].valid, __ATOMIC_ACQUIRE)) {
+    hipDeviceProp_t p;
+    MS_HIP(hipGetDeviceProperties(&p, d));
+    g_dev[d].cus = p.multiProcessorCount;
+    g_dev[d].clock_khz = p.clockRate;
+    g_dev[d].gfx950 = strncmp(p.gcnArchName, "gfx950", 6) == 0;
+    g_dev[d].lds = (int)p.sharedMemPerBlock;
+    __atomic_store_n(&g_dev[d].valid, 1, __ATOMIC_RELEASE);
+  }
+  *out = &g_dev[d];
+  return MS_OK;
+}
+
+enum Flow { OS = 0, LS = 1, RS = 2 };
+
+// One local contraction, in kernel terms.
+struct Problem {
+  Flow flow;
+  const void *const *a;  // nkslices (OS) or nchunks (RS) or 1 pointers
+  const void *const *b;
+  void *const *c;
+  int na, nb, nc;
+  int S;
+  int M, N, K;           // per-chunk rows/cols, per-slice contraction
+  int lda, ldb, ldc;
+  int in_dtype, out_dtype;
+};
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int validate(const Problem &p) {
+  static const char *names[] = {"ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs"};
+  const char *fn = names[p.flow];
+  if (p.S < 1 || p.S > MS_MAX_SLICES) return fail(MS_ERR_ARG, "%s: S = %d outside [1, %d]", fn, p.S, MS_MAX_SLICES);
+  if (p.M <= 0 || p.N <= 0 || p.K <= 0) return fail(MS_ERR_ARG, "%s: non-positive extent (m=%d n=%d k=%d)", fn, p.M, p.N, p.K);
+  if (p.in_dtype != MS_DTYPE_F32 && p.in_dtype != MS_DTYPE_BF16) return fail(MS_ERR_UNSUPPORTED, "%s: unknown in_dtype %d", fn, p.in_dtype);
+  if (p.out_dtype != MS_DTYPE_F32 && p.out_dtype != MS_DTYPE_BF16) return fail(MS_ERR_UNSUPPORTED, "%s: unknown out_dtype %d", fn, p.out_dtype);
+  if (!p.a || !p.b || !p.c) return fail(MS_ERR_ARG, "%s: null pointer table", fn);
+  const int q = p.in_dtype == MS_DTYPE_BF16 ? 8 : 4;  // elements per 16 bytes
+  // contiguous extent of each operand, and minimum leading dimension
+  const int a_cont = p.flow == RS ? p.M : p.K;
+  const int b_cont = p.flow == LS ? p.K : p.N;
+  if (a_cont % q || b_cont % q) return fail(MS_ERR_ARG, "%s: contiguous extents (%d, %d) must be multiples of %d", fn, a_cont, b_cont, q);
+  if (p.lda < a_cont || p.ldb < b_cont || p.ldc < p.N) return fail(MS_ERR_ARG, "%s: leading dimension smaller than the row length", fn);
+  if (p.lda % q || p.ldb % q) return fail(MS_ERR_ARG, "%s: operand leading dimensions must be multiples of %d", fn, q);
+  const int qo = p.out_dtype == MS_DTYPE_BF16 ? 8 : 4;
+  if (p.N % qo || p.ldc % qo) return fail(MS_ERR_ARG, "%s: output columns / leading dimension must be multiples of %d", fn, qo);
+  for (int i = 0; i < p.na; i++) if (!p.a[i] || !aligned16(p.a[i])) return fail(MS_ERR_ARG, "%s: operand pointer %d null or not 16-byte aligned", fn, i);
+  for (int i = 0; i < p.nb; i++) if (!p.b[i] || !aligned16(p.b[i])) return fail(MS_ERR_ARG, "%s: operand pointer %d null or not 16-byte aligned", fn, i);
+  for (int i = 0; i < p.nc; i++) if (!p.c[i] || !aligned16(p.c[i])) return fail(MS_ERR_ARG, "%s: output pointer %d null or not 16-byte aligned", fn, i);
+  return MS_OK;
+}
+
+template <int BM, int BN, int WGM, int WGN, bool AK, bool BK_, bool OBF>
+void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
+  msk::gemm_bf16_kernel<BM, BN, WGM, WGN, AK, BK_, OBF><<<gd, bd, 0, stream>>>(g);
+}
+
+template <int BM, int BN, int WGM, int WGN>
+int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+  msk::GemmArgs g;
+  memset(&g, 0, sizeof(g));
+  for (int i = 0; i < p.na; i++) g.a[i] = p.a[i];
+  for (int i = 0; i < p.nb; i++) g.b[i] = p.b[i];
+  for (int i = 0; i < p.nc; i++) g.c[i] = p.c[i];
+  g.nchunks = p.flow == OS ? 1 : p.S;
+  g.nkslices = p.flow == OS ? p.S : 1;
+  g.a_by_chunk = p.flow == RS;
+  g.b_by_chunk = p.flow == LS;
+  g.M = p.M; g.N = p.N; g.K = p.K;
+  g.lda = p.lda; g.ldb = p.ldb; g.ldc = p.ldc;
+  g.tiles_m = (p.M + BM - 1) / BM;
+  g.tiles_n = (p.N + BN - 1) / BN;
+  const long total = (long)g.tiles_m * g.tiles_n * g.nchunks;
+  if (total > 0x7FFFFFFF) return fail(MS_ERR_ARG, "problem has too many tiles");
+  g.total_tiles = (int)total;
+  g.group_m = 8;
+  int grid = dev.cus < g.total_tiles ? dev.cus : g.total_tiles;
+  dim3 gd(grid), bd(WGM * WGN * 64);
+  const bool obf = p.out_dtype == MS_DTYPE_BF16;
+  if (p.flow == OS) {
+    if (obf) launch_one<BM, BN, WGM, WGN, true, false, true>(gd, bd, stream, g);
+    else launch_one<BM, BN, WGM, WGN, true, false, false>(gd, bd, stream, g);
+  } else if (p.flow == LS) {
+    launch_one<BM, BN, WGM, WGN, true, true, false>(gd, bd, stream, g);
+  } else {
+    launch_one<BM, BN, WGM, WGN, false, false, false>(gd, bd, stream, g);
+  }
+  MS_HIP(hipGetLastError());
+  return MS_OK;
+}
+
+int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+  if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
+  int v = g_variant;
+  if (v == 0) {
+    // small outputs cannot fill 256 CUs with 256x256 tiles
+    const long t256 = (long)((p.M + 255) / 256) * ((p.N + 255) / 256) * (p.flow == OS ? 1 : p.S);
+    v = t256 >= dev.cus ? 1 : 3;
+  }
+  switch (v) {
+    case 1: return launch_bf16_tile<256, 256, 2, 2>(p, dev, stream);
+    case 2: return launch_bf16_tile<256, 256, 2, 4>(p, dev, stream);
+    case 3: return launch_bf16_tile<128, 128, 2, 2>(p, dev, stream);
+    default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
+  }
+}
+
+int launch_f32(const Problem &p, hipStream_t stream) {
+  msk::GemmArgsF32 g;
+  memset(&g, 0, sizeof(g));
+  for (int i = 0; i < p.na; i++) g.a[i] = p.a[i];
+  for (int i = 0; i < p.nb; i++) g.b[i] = p.b[i];
+  for (int i = 0; i < p.nc; i++) g.c[i] = p.c[i];
+  g.nchunks = p.flow == OS ? 1 : p.S;
+  g.nkslices = p.flow == OS ? p.S : 1;
+  g.a_by_chunk = p.flow == RS;
+  g.b_by_chunk = p.flow == LS;
+  g.M = p.M; g.N = p.N; g.K = p.K;
+  if (p.flow == RS) { g.a_rs = 1; g.a_cs = p.lda; } else { g.a_rs = p.lda; g.a_cs = 1; }
+  if (p.flow == LS) { g.b_rs = 1; g.b_cs = p.ldb; } else { g.b_rs = p.ldb; g.b_cs = 1; }
+  g.ldc = p.ldc;
+  g.tiles_m = (p.M + 63) / 64;
+  g.tiles_n = (p.N + 63) / 64;
+  const long total = (long)g.tiles_m * g.tiles_n * g.nchunks;
+  if (total > 0x7FFFFFFF) return fail(MS_ERR_ARG, "problem has too many tiles");
+  dim3 gd((unsigned)total), bd(256);
+  if (p.out_dtype == MS_DTYPE_BF16) hipLaunchKernelGGL(msk::gemm_f32_kernel<true>, gd, bd, 0, stream, g);
+  else hipLaunchKernelGGL(msk::gemm_f32_kernel<false>, gd, bd, 0, stream, g);
+  MS_HIP(hipGetLastError());
+  return MS_OK;
+}
+
+int run(const Problem &p, void *stream) {
+  int rc = validate(p);
+  if (rc) return rc;
+  DevInfo *dev = nullptr;
+  rc = dev_info(&dev);
+  if (rc) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  return p.in_dtype == MS_DTYPE_BF16 ? launch_bf16(p, *dev, st) : launch_f32(p, st);
+}
+
+int timed(const Problem &p, void *stream, int warmup, int reps, float *ms_out) {
+  if (warmup < 0 || reps < 1 || !ms_out) return fail(MS_ERR_ARG, "timing: need warmup >= 0, reps >= 1 and an output array");
+  hipStream_t st = (hipStream_t)stream;
+  for (int i = 0; i < warmup; i++) {
+    int rc = run(p, stream);
+    if (rc) return rc;
+  }
+  hipEvent_t e0, e1;
+  MS_HIP(hipEventCreate(&e0));
+  MS_HIP(hipEventCreate(&e1));
+  int rc = MS_OK;
+  for (int r = 0; r < reps && rc == MS_OK; r++) {
+    (void)hipEventRecord(e0, st);
+    rc = run(p, stream);
+    (void)hipEventRecord(e1, st);
+    if (hipEventSynchronize(e1) != hipSuccess) rc = fail(MS_ERR_HIP, "hipEventSynchronize failed");
+    float ms = 0.f;
+    if (rc == MS_OK && hipEventElapsedTime(&ms, e0, e1) != hipSuccess) rc = fail(MS_ERR_HIP, "hipEventElapsedTime failed");
+    ms_out[r] = ms;
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc == MS_OK) MS_HIP(hipStreamSynchronize(st));
+  return rc;
+}
+
+Problem make_os(const void *const *A, const void *const *B, int S, int m, int n, int k, int lda, int ldb,
+                void *const *C, int ldc, int in_dtype, int out_dtype) {
+  Problem p{OS, A, B, C, S, S, 1, S, m, n, k, lda, ldb, ldc, in_dtype, out_dtype};
+  if (S < 1 || S > MS_MAX_SLICES) p.na = p.nb = 0;
+  return p;
+}
+Problem make_ls(const void *const *A, int lda, const void *const *W, int ldw, int S, int m, int n, int k,
+                float *const *Y, int ldy, int in_dtype) {
+  Problem p{LS, A, W, (void *const *)Y, 1, S, S, S, m, n, k, lda, ldw, ldy, in_dtype, MS_DTYPE_F32};
+  if (S < 1 || S > MS_MAX_SLICES) p.nb = p.nc = 0;
+  return p;
+}
+Problem make_rs(const void *const *X, int ldx, const void *const *W, int ldw, int S, int m, int n, int k,
+                float *const *Y, int ldy, int in_dtype) {
+  Problem p{RS, X, W, (void *const *)Y, S, 1, S, S, m, n, k, ldx, ldw, ldy, in_dtype, MS_DTYPE_F32};
+  if (S < 1 || S > MS_MAX_SLICES) p.na = p.nc = 0;
+  return p;
+}
+
+}  // namespace
+
+MS_API int ms_version(void) { return 100; }
+
+MS_API const char *ms_last_error(void) { return g_err; }
+
+MS_API long ms_query(int what) {
+  if (what == MS_QUERY_MAX_SLICES) return MS_MAX_SLICES;
+  DevInfo *d = nullptr;
+  if (dev_info(&d) != MS_OK) return -1;
+  switch (what) {
+    case MS_QUERY_CU_COUNT: return d->cus;
+    case MS_QUERY_CLOCK_KHZ: return d->clock_khz;
+    case MS_QUERY_IS_GFX950: return d->gfx950;
+    case MS_QUERY_LDS_BYTES: return d->lds;
+    default: fail(MS_ERR_ARG, "ms_query: unknown selector %d", what); return -1;
+  }
+}
+
+MS_API int ms_set_variant(int variant) {
+  if (variant < 0 || variant > 3) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  g_variant = variant;
+  return MS_OK;
+}
+
+MS_API int ms_gemm_os(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
+                      int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype, void *stream) {
+  void *c1[1] = {C};
+  return run(make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype), stream);
+}
+
+MS_API int ms_gemm_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
+                      float *const *Y_chunks, int ldy, int in_dtype, void *stream) {
+  const void *a1[1] = {A};
+  return run(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, Y_chunks, ldy, in_dtype), stream);
+}
+
+MS_API int ms_gemm_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
+                      float *const *Y_chunks, int ldy, int in_dtype, void *stream) {
+  const void *w1[1] = {W};
+  return run(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype), stream);
+}
+
+MS_API int ms_time_os(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
+                      int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype, void *stream,
+                      int warmup, int reps, float *ms_out) {
+  void *c1[1] = {C};
+  return timed(make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype), stream, warmup, reps, ms_out);
+}
+
+MS_API int ms_time_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
+                      float *const *Y_chunks, int ldy, int in_dtype, void *stream, int warmup, int reps, float *ms_out) {
+  const void *a1[1] = {A};
+  return timed(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, Y_chunks, ldy, in_dtype), stream, warmup, reps, ms_out);
+}
+
+MS_API int ms_time_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
+                      float *const *Y_chunks, int ldy, int in_dtype, void *stream, int warmup, int reps, float *ms_out) {
+  const void *w1[1] = {W};
+  return timed(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype), stream, warmup, reps, ms_out);
+}

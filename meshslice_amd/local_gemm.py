@@ -1,0 +1,142 @@
+"""The per-device local contraction of the three dataflows on torch device tensors.
+
+These functions are what the per-device bodies in TensorParallel.py call where the reference calls
+``jnp.einsum`` / ``@`` (reference TensorParallel.py:22,26,31,162,167,172,181,187,203,209).  torch is
+used only to own device memory and to name the current stream; all arithmetic happens in
+libmeshslice_hip.so.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.MS_DTYPE_F32, torch.bfloat16: _lib.MS_DTYPE_BF16}
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype not in _DT:
+        raise TypeError(f"unsupported dtype {t.dtype}: the local GEMM takes float32 or bfloat16")
+    return _DT[t.dtype]
+
+
+def _check2d(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise _lib.MeshSliceError(f"{name} is not on the GPU: the local GEMM has no CPU path")
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise ValueError(f"{name} must be a row-major 2-D tensor (got shape {tuple(t.shape)}, strides {t.stride()})")
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _same(ts: Sequence[torch.Tensor], name: str):
+    if len(ts) < 1:
+        raise ValueError(f"{name}: need at least one slice")
+    s0 = ts[0]
+    for t in ts:
+        _check2d(t, name)
+        if t.shape != s0.shape or t.dtype != s0.dtype or t.stride(0) != s0.stride(0) or t.device != s0.device:
+            raise ValueError(f"{name}: all slices must share shape, dtype, leading dimension and device")
+    return s0
+
+
+def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
+            out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """``C = sum_s A_s @ B_s`` with fp32 accumulation over all slices, rounded once."""
+    a0 = _same(A_slices, "A_slices"); b0 = _same(B_slices, "B_slices")
+    if len(A_slices) != len(B_slices):
+        raise ValueError("A_slices and B_slices differ in length")
+    if a0.shape[1] != b0.shape[0] or a0.dtype != b0.dtype:
+        raise ValueError(f"slice shapes do not contract: {tuple(a0.shape)} @ {tuple(b0.shape)}")
+    m, k = a0.shape; n = b0.shape[1]
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype or a0.dtype, device=a0.device)
+    _check2d(out, "out")
+    if tuple(out.shape) != (m, n):
+        raise ValueError("out has the wrong shape")
+    pa, _ka = _lib.ptr_array([t.data_ptr() for t in A_slices])
+    pb, _kb = _lib.ptr_array([t.data_ptr() for t in B_slices])
+    with torch.cuda.device(a0.device):
+        rc = _lib.load().ms_gemm_os(pa, pb, len(A_slices), m, n, k, a0.stride(0), b0.stride(0),
+                                    ctypes.c_void_p(out.data_ptr()), out.stride(0), _dt(a0), _dt(out), _stream())
+    _lib.check(rc)
+    return out
+
+
+def gemm_ls(A: torch.Tensor, W_slices: Sequence[torch.Tensor],
+            out: Optional[List[torch.Tensor]] = None) -> List[torch.Tensor]:
+    """``Y_s = A @ W_s^T`` (fp32 chunks), W_s stored ``[n_slice, k]``."""
+    _check2d(A, "A"); w0 = _same(W_slices, "W_slices")
+    if A.shape[1] != w0.shape[1] or A.dtype != w0.dtype:
+        raise ValueError(f"shapes do not contract: {tuple(A.shape)} @ {tuple(w0.shape)}^T")
+    m, k = A.shape; ns = w0.shape[0]; S = len(W_slices)
+    if out is None:
+        buf = torch.empty((S, m, ns), dtype=torch.float32, device=A.device)
+        out = [buf[s] for s in range(S)]
+    o0 = _same(out, "out")
+    if len(out) != S or tuple(o0.shape) != (m, ns) or o0.dtype != torch.float32:
+        raise ValueError("out must be S fp32 chunks of shape [m, n_slice]")
+    pw, _kw = _lib.ptr_array([t.data_ptr() for t in W_slices])
+    py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
+    with torch.cuda.device(A.device):
+        rc = _lib.load().ms_gemm_ls(ctypes.c_void_p(A.data_ptr()), A.stride(0), pw, w0.stride(0), S, m, ns, k,
+                                    py, o0.stride(0), _dt(A), _stream())
+    _lib.check(rc)
+    return list(out)
+
+
+def gemm_rs(X_slices: Sequence[torch.Tensor], W: torch.Tensor,
+            out: Optional[List[torch.Tensor]] = None) -> List[torch.Tensor]:
+    """``Y_s = X_s^T @ W`` (fp32 chunks), X_s stored ``[k, m_slice]``."""
+    _check2d(W, "W"); x0 = _same(X_slices, "X_slices")
+    if x0.shape[0] != W.shape[0] or x0.dtype != W.dtype:
+        raise ValueError(f"shapes do not contract: {tuple(x0.shape)}^T @ {tuple(W.shape)}")
+    k, ms = x0.shape; n = W.shape[1]; S = len(X_slices)
+    if out is None:
+        buf = torch.empty((S, ms, n), dtype=torch.float32, device=W.device)
+        out = [buf[s] for s in range(S)]
+    o0 = _same(out, "out")
+    if len(out) != S or tuple(o0.shape) != (ms, n) or o0.dtype != torch.float32:
+        raise ValueError("out must be S fp32 chunks of shape [m_slice, n]")
+    px, _kx = _lib.ptr_array([t.data_ptr() for t in X_slices])
+    py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
+    with torch.cuda.device(W.device):
+        rc = _lib.load().ms_gemm_rs(px, x0.stride(0), ctypes.c_void_p(W.data_ptr()), W.stride(0), S, ms, n, k,
+                                    py, o0.stride(0), _dt(W), _stream())
+    _lib.check(rc)
+    return list(out)
+
+
+def time_call(flow: str, operands, out, warmup: int = 5, reps: int = 20) -> List[float]:
+    """Per-launch milliseconds (HIP events on the current stream) of one local contraction.
+
+    ``flow`` is 'os', 'ls' or 'rs'; ``operands``/``out`` are what gemm_os/gemm_ls/gemm_rs take."""
+    ms = (ctypes.c_float * reps)()
+    lib = _lib.load()
+    if flow == "os":
+        A, B = operands
+        pa, _ka = _lib.ptr_array([t.data_ptr() for t in A]); pb, _kb = _lib.ptr_array([t.data_ptr() for t in B])
+        m, k = A[0].shape; n = B[0].shape[1]
+        rc = lib.ms_time_os(pa, pb, len(A), m, n, k, A[0].stride(0), B[0].stride(0), ctypes.c_void_p(out.data_ptr()),
+                            out.stride(0), _dt(A[0]), _dt(out), _stream(), warmup, reps, ms)
+    elif flow == "ls":
+        A, W = operands
+        pw, _kw = _lib.ptr_array([t.data_ptr() for t in W]); py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
+        m, k = A.shape; ns = W[0].shape[0]
+        rc = lib.ms_time_ls(ctypes.c_void_p(A.data_ptr()), A.stride(0), pw, W[0].stride(0), len(W), m, ns, k,
+                            py, out[0].stride(0), _dt(A), _stream(), warmup, reps, ms)
+    elif flow == "rs":
+        X, W = operands
+        px, _kx = _lib.ptr_array([t.data_ptr() for t in X]); py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
+        k, msl = X[0].shape; n = W.shape[1]
+        rc = lib.ms_time_rs(px, X[0].stride(0), ctypes.c_void_p(W.data_ptr()), W.stride(0), len(X), msl, n, k,
+                            py, out[0].stride(0), _dt(W), _stream(), warmup, reps, ms)
+    else:
+        raise ValueError(f"unknown dataflow {flow!r}")
+    _lib.check(rc)
+    return list(ms)
