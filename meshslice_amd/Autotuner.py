@@ -1,0 +1,165 @@
+"""The parts of the reference's autotuner that consume the measured compute term.
+
+* ``FFLayerModel`` with its dataflow rule and ``emulate`` (reference Autotuner.py:21-35, :141-169):
+  forward + backward-data + backward-weight model time of one feed-forward layer for a slice count;
+* ``possibleK`` (:242-273): admissible slice counts from the divisibility of the sliced extent;
+* ``emulateFFTime`` (:391-426): per layer, scan the candidate slice counts and keep the best;
+* the interconnect constants the reference measured on TPUv4 (:17-19), kept as data;
+* ``sweep_compute_term``: time the per-slice kernels of one GPT-3-like layer on the MI355X for
+  several meshes and slice counts and refit ``CostModel.estimateMatmul``'s compute term.
+
+The graph builder, transposition pass and analytical mesh search of the reference are host
+bookkeeping with no device work and are not built.  Two slips of the reference are not reproduced:
+``emulateFFTime`` records the loop variable of the scan as the best slice count (the reference
+stores the module-level ``K``, :418), and an unknown dataflow name is an error.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Iterable, List, Sequence, Tuple
+
+from . import CostModel
+from .CostModel import DeviceMesh
+
+# TPUv4 interconnect calibration shipped with the reference (Autotuner.py:17-19)
+latencies = {"allgather": 5e-6, "reducescatter": 5e-6, "sendrecv": 5e-5}
+bws = {"allgather": (27.472e9, 79.751e9), "reducescatter": (37.506e9, 63.167e9), "sendrecv": (38.801e9, 35.224e9)}
+base_overheads = {"allgather": 13e-6, "reducescatter": 26e-6, "sendrecv": 13e-6}
+
+
+def default_mesh(shape, flops: float = CostModel.BF16_PEAK_FLOPS) -> DeviceMesh:
+    return DeviceMesh(shape, flops, bws_per_direction=bws, link_latencies=latencies, base_overheads=base_overheads)
+
+
+def pick_dataflow(B: int, I: int, O: int) -> str:
+    """Keep the largest of (tokens x in, tokens x out, in x out) stationary (reference :29-34, :297-302)."""
+    if O > I and B >= I:
+        return "os"
+    if I >= O and B >= O:
+        return "ls"
+    return "rs"
+
+
+class FFLayerModel:
+    def __init__(self, B, I, O, dataflow=None, transpose=False):
+        self.bsize, self.in_dim, self.out_dim = B, I, O
+        if dataflow is None:
+            dataflow = pick_dataflow(B, I, O)
+        if dataflow not in ("os", "ls", "rs"):
+            raise ValueError(f"unknown dataflow {dataflow!r}")
+        self.dataflow = dataflow
+        self.transpose = transpose
+
+    def passes(self) -> List[Tuple[str, int, int, int]]:
+        """(model, M, N, K) of the forward, backward-data and backward-weight GEMMs (reference :142-167)."""
+        B, I, O = self.bsize, self.in_dim, self.out_dim
+        plain = {
+            "os": [("os", B, O, I), ("ls", B, I, O), ("rs", I, O, B)],
+            "ls": [("ls", B, O, I), ("os", B, I, O), ("rs", O, I, B)],
+            "rs": [("rs", B, O, I), ("ls", I, B, O), ("os", I, O, B)],
+        }
+        transposed = {
+            "os": [("os", O, B, I), ("rs", I, B, O), ("ls", O, I, B)],
+            "ls": [("rs", O, B, I), ("os", I, B, O), ("ls", I, O, B)],
+            "rs": [("ls", O, B, I), ("rs", B, I, O), ("os", O, I, B)],
+        }
+        return (transposed if self.transpose else plain)[self.dataflow]
+
+    def emulate(self, mesh: DeviceMesh, K: int) -> float:
+        model = {"os": CostModel.MeshFlow_OS, "ls": CostModel.MeshFlow_LS, "rs": CostModel.MeshFlow_RS}
+        total = 0.0
+        for name, M, N, Kd in self.passes():
+            pro, steady = model[name](mesh, M, N, Kd, K)
+            total += pro + steady
+        return total
+
+
+def possibleK(B, I, O, meshshape, dataflow) -> List[int]:
+    """Candidate slice counts (reference :242-273): the sliced extent, divided by lcm(R, C) and by the
+    block size 8, picks a list by its divisibility."""
+    mlcm = meshshape[0] * meshshape[1] // math.gcd(meshshape[0], meshshape[1])
+    kdim = {"os": I, "ls": O}.get(dataflow, B) // mlcm // 8
+    ladder = [(48, [3, 4, 6, 8, 12, 16, 24]), (40, [4, 5, 8, 10, 20]), (24, [3, 4, 6, 8, 12, 24]),
+              (20, [4, 5, 10, 20]), (16, [4, 8, 16]), (12, [3, 4, 12]), (10, [5, 10]), (8, [4, 8]),
+              (6, [3, 6]), (4, [4]), (5, [5])]
+    for div, ks in ladder:
+        if kdim % div == 0:
+            return list(ks)
+    return [kdim]
+
+
+def emulateFFTime(layers: Sequence[Tuple[int, int, int, str]], meshshape, sweep: bool = False,
+                  candidates=None, verbose: bool = False):
+    """Model time of the feed-forward layers ``(B, I, O, dataflow)`` on ``meshshape`` with the best slice
+    count per layer (reference :391-426).  Without ``sweep`` the scan stops at the first slice count
+    that does not improve.  Returns ``(seconds, [best K per layer])``."""
+    mesh = default_mesh(meshshape)
+    total, best = 0.0, []
+    for (B, I, O, dataflow) in layers:
+        model = FFLayerModel(B, I, O, dataflow)
+        klist = list(candidates) if candidates is not None else possibleK(B, I, O, meshshape, dataflow)
+        bestK, bestT = klist[0], model.emulate(mesh, klist[0])
+        for k in klist[1:]:
+            t = model.emulate(mesh, k)
+            if verbose:
+                print(f"FFtime at k={k} is {t}")
+            if t < bestT:
+                bestK, bestT = k, t
+            elif not sweep:
+                break
+        total += bestT
+        best.append(bestK)
+    return total, best
+
+
+# ------------------------------------------------------------------------------------------------
+# compute-term sweep on the MI355X
+# ------------------------------------------------------------------------------------------------
+
+def gpt3_layers(tokens: int = 16384, hidden: int = 12288, ffn: int = 49152) -> List[Tuple[str, int, int, int, str]]:
+    """(name, B, I, O, dataflow) of the four feed-forward GEMMs of one GPT-3-like layer, with the
+    dataflows the reference's benchmark assigns (BenchTransformer.py:80-93)."""
+    return [("in_proj", tokens, hidden, 3 * hidden, "os"), ("out_proj", tokens, hidden, hidden, "ls"),
+            ("ff1", tokens, hidden, ffn, "os"), ("ff2", tokens, ffn, hidden, "ls")]
+
+
+def per_slice_shapes(B, I, O, dataflow, meshshape, S, passes=("fwd", "bwd_data", "bwd_weight")):
+    """Per-slice kernel shapes ``(pass, M, N, K, layout)`` a device runs, by the rules of
+    CostModel.MeshFlow_OS/LS/RS: OS (M/R, N/C, K/S) nn; LS (M/R, N/S, K/C) nt; RS (M/S, N/C, K/R) tn."""
+    R, C = meshshape
+    out = []
+    names = ("fwd", "bwd_data", "bwd_weight")
+    for pname, (model, M, N, K) in zip(names, FFLayerModel(B, I, O, dataflow).passes()):
+        if pname not in passes:
+            continue
+        if model == "os":
+            out.append((pname, M // R, N // C, K // S, "nn"))
+        elif model == "ls":
+            out.append((pname, M // R, N // S, K // C, "nt"))
+        else:
+            out.append((pname, M // S, N // C, K // R, "tn"))
+    return out
+
+
+def sweep_compute_term(meshes=((2, 8), (4, 4), (8, 8)), slice_counts=(1, 2, 4, 8, 16),
+                       passes=("fwd",), layers=None, repeat: int = 5, verbose: bool = True):
+    """Measure every per-slice kernel of the sweep on the GPU and fit the compute term.
+
+    Returns ``(ComputeTerm, rows)`` where each row is
+    ``(mesh, layer, pass, S, M, N, K, layout, seconds_per_slice)``."""
+    layers = layers or gpt3_layers()
+    rows, samples, seen = [], [], {}
+    for mesh in meshes:
+        for (lname, B, I, O, dataflow) in layers:
+            for S in slice_counts:
+                for (pname, M, N, K, layout) in per_slice_shapes(B, I, O, dataflow, mesh, S, passes):
+                    key = (M, N, K, layout)
+                    if key not in seen:
+                        seen[key] = CostModel.estimateMatmul(None, M, N, K, layout=layout, repeat=repeat)
+                        samples.append((M, N, K, layout, seen[key]))
+                    rows.append((mesh, lname, pname, S, M, N, K, layout, seen[key]))
+                    if verbose:
+                        tf = 2.0 * M * N * K / seen[key] / 1e12
+                        print(f"mesh {mesh[0]}x{mesh[1]} {lname:8s} {pname:10s} S={S:2d} {layout} "
+                              f"[{M}x{N}x{K}] {seen[key]*1e3:.4f} ms/slice {tf:.0f} TFLOP/s", flush=True)
+    return CostModel.fit_compute_term(samples), rows

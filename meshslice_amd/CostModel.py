@@ -1,0 +1,239 @@
+"""Time model of the 2-D GEMM algorithms: analytical communication terms plus a MEASURED compute term.
+
+Follows reference CostModel.py: ``DeviceMesh`` (:8-29), the ring all-gather / reduce-scatter
+estimates (:47-63, :120-134), ``estimateMatmul`` (:74-98), the unsliced ``GSPMD_OS/LS/RS`` (:220-247)
+and the sliced ``MeshFlow_OS/LS/RS`` (:249-285) models, each returning ``(prologue, steady_state)``
+seconds.  The SUMMA / Cannon / logical-ring models of the reference are comparison baselines and are
+not built.
+
+The compute term is what this build changes: ``estimateMatmul`` times the gfx950 kernel of the same
+layout on the MI355X (HIP events, one warm-up + ``repeat`` launches, mean), or — when a fitted
+``ComputeTerm`` has been installed with ``use_compute_term`` — evaluates ``t0 + 2MNK / (eta * peak)``
+without touching the GPU.  There is no CPU timing path.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Iterable, Optional, Tuple
+
+import numpy as np
+
+BF16_PEAK_FLOPS = 2.5166e15   # MI355X dense bf16 MFMA peak: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
+
+
+class DeviceMesh:
+    """Mesh shape + link parameters (reference CostModel.py:8-29).  One of the two extents may itself
+    be a pair ``(r, c)``: that mesh dimension is then a 2-D sub-mesh of r*c devices."""
+
+    def __init__(self, device_shape: tuple, flops_per_chip: float, bws_per_direction, link_latencies, base_overheads):
+        self.reshape(device_shape)
+        self.flops = flops_per_chip
+        self.bws = bws_per_direction
+        self.link_latencies = link_latencies
+        self.base_overheads = base_overheads
+
+    def reshape(self, newshape):
+        self.meshdim = None
+        self.submesh = None
+        dims = []
+        for d, ext in enumerate(newshape):
+            if isinstance(ext, tuple):
+                self.meshdim, self.submesh = d, ext
+                dims.append(ext[0] * ext[1])
+            else:
+                dims.append(ext)
+        self.shape = tuple(dims)
+
+
+def bytesize(shape) -> int:
+    return shape[0] * shape[1] * 2
+
+
+def _ring_collective(mesh: DeviceMesh, kind: str, data_shape, dim: int, precision: int) -> float:
+    """Ring all-gather / reduce-scatter along mesh dimension ``dim``: ``size-1`` steps, each moving one
+    shard and paying one link latency, plus a fixed launch overhead.  On a sub-meshed dimension the
+    two halves of the data travel row-first and column-first at once (reference :55-62, :127-133)."""
+    nbytes = data_shape[0] * data_shape[1] * precision // 8
+    lat = mesh.link_latencies[kind]
+    base = mesh.base_overheads[kind]
+    bw = mesh.bws[kind][dim]
+    if mesh.meshdim is not None and dim == mesh.meshdim:
+        r, c = mesh.submesh
+        half = nbytes // 2
+        row_first = (half / bw) * (r - 1) + (half * r / bw) * (c - 1)
+        col_first = (half / bw) * (c - 1) + (half * c / bw) * (r - 1)
+        return base + max(row_first, col_first) + lat * (r + c - 2)
+    steps = mesh.shape[dim] - 1
+    return base + steps * (nbytes / bw) + lat * steps
+
+
+def estimateAllgather(mesh: DeviceMesh, data_shape: tuple, dim: int, precision: int) -> float:
+    return _ring_collective(mesh, "allgather", data_shape, dim, precision)
+
+
+def estimateReduceScatter(mesh: DeviceMesh, data_shape: tuple, dim: int, precision: int) -> float:
+    return _ring_collective(mesh, "reducescatter", data_shape, dim, precision)
+
+
+# ------------------------------------------------------------------------------------------------
+# compute term
+# ------------------------------------------------------------------------------------------------
+
+@dataclass
+class ComputeTerm:
+    """Fitted model of one kernel launch: ``t = t0 + 2*M*N*K / (eta * peak)`` per layout, with the
+    measured points kept for exact look-up."""
+    t0: Dict[str, float] = field(default_factory=dict)
+    eta: Dict[str, float] = field(default_factory=dict)
+    table: Dict[Tuple[int, int, int, str], float] = field(default_factory=dict)
+    peak: float = BF16_PEAK_FLOPS
+
+    def seconds(self, M: int, N: int, K: int, layout: str) -> float:
+        hit = self.table.get((int(M), int(N), int(K), layout))
+        if hit is not None:
+            return hit
+        if layout not in self.eta:
+            raise KeyError(f"no fitted compute term for layout {layout!r}")
+        return self.t0[layout] + 2.0 * M * N * K / (self.eta[layout] * self.peak)
+
+    def to_dict(self):
+        return {"peak": self.peak, "t0": self.t0, "eta": self.eta,
+                "table": [[m, n, k, lay, t] for (m, n, k, lay), t in sorted(self.table.items())]}
+
+    @classmethod
+    def from_dict(cls, d):
+        ct = cls(t0=dict(d["t0"]), eta=dict(d["eta"]), peak=float(d.get("peak", BF16_PEAK_FLOPS)))
+        for m, n, k, lay, t in d.get("table", []):
+            ct.table[(int(m), int(n), int(k), lay)] = float(t)
+        return ct
+
+
+def fit_compute_term(samples: Iterable[Tuple[int, int, int, str, float]], peak: float = BF16_PEAK_FLOPS) -> ComputeTerm:
+    """Least-squares fit of ``t = t0 + flops / (eta*peak)`` per layout from measured
+    ``(M, N, K, layout, seconds)`` samples."""
+    ct = ComputeTerm(peak=peak)
+    by_layout: Dict[str, list] = {}
+    for m, n, k, lay, t in samples:
+        ct.table[(int(m), int(n), int(k), lay)] = float(t)
+        by_layout.setdefault(lay, []).append((2.0 * m * n * k, float(t)))
+    for lay, pts in by_layout.items():
+        f = np.array([p[0] for p in pts]); t = np.array([p[1] for p in pts])
+        if len(pts) >= 2 and np.ptp(f) > 0:
+            slope, icpt = np.polyfit(f, t, 1)
+        else:
+            slope, icpt = t[0] / f[0], 0.0
+        if slope <= 0:   # degenerate sample set: fall back to the mean rate
+            slope, icpt = float(np.sum(t) / np.sum(f)), 0.0
+        ct.t0[lay] = float(max(icpt, 0.0))
+        ct.eta[lay] = float(1.0 / (slope * peak))
+    return ct
+
+
+_installed: Optional[ComputeTerm] = None
+_measured: Dict[tuple, float] = {}
+
+
+def use_compute_term(term: Optional[ComputeTerm]) -> None:
+    """Install (or, with None, remove) a fitted compute term used by ``estimateMatmul``."""
+    global _installed
+    _installed = term
+
+
+def estimateMatmul(mesh, M, N, K, input_precision=None, layout: str = "nn", repeat: int = 5) -> float:
+    """Seconds of one local ``[M,K] x [K,N]`` contraction (reference CostModel.py:74-98).
+
+    ``layout``: 'nn' (OS slice), 'nt' (LS: B stored [N,K]), 'tn' (RS: A stored [K,M]).  ``mesh`` is
+    unused, as in the reference.  Measures on the GPU unless a fitted term is installed."""
+    if layout not in ("nn", "nt", "tn"):
+        raise ValueError(f"unknown layout {layout!r}")
+    M, N, K = int(M), int(N), int(K)
+    if _installed is not None:
+        return _installed.seconds(M, N, K, layout)
+    import torch
+    from . import local_gemm
+    dtype = input_precision or torch.bfloat16
+    key = (M, N, K, layout, dtype, repeat)
+    if key in _measured:
+        return _measured[key]
+    if not torch.cuda.is_available():
+        raise local_gemm._lib.MeshSliceError(
+            "estimateMatmul needs the GPU (or a fitted ComputeTerm installed with use_compute_term)")
+    dev = "cuda"
+    if layout == "nn":
+        A = torch.ones((M, K), dtype=dtype, device=dev); B = torch.ones((K, N), dtype=dtype, device=dev)
+        out = torch.empty((M, N), dtype=dtype, device=dev)
+        ms = local_gemm.time_call("os", ([A], [B]), out, warmup=1, reps=repeat)
+    elif layout == "nt":
+        A = torch.ones((M, K), dtype=dtype, device=dev); B = torch.ones((N, K), dtype=dtype, device=dev)
+        out = [torch.empty((M, N), dtype=torch.float32, device=dev)]
+        ms = local_gemm.time_call("ls", (A, [B]), out, warmup=1, reps=repeat)
+    else:
+        A = torch.ones((K, M), dtype=dtype, device=dev); B = torch.ones((K, N), dtype=dtype, device=dev)
+        out = [torch.empty((M, N), dtype=torch.float32, device=dev)]
+        ms = local_gemm.time_call("rs", ([A], B), out, warmup=1, reps=repeat)
+    sec = float(np.mean(ms)) * 1e-3
+    _measured[key] = sec
+    return sec
+
+
+# ------------------------------------------------------------------------------------------------
+# algorithm models: (prologue, steady state)
+# ------------------------------------------------------------------------------------------------
+
+def GSPMD_OS(mesh, M, N, K, steps=8, precisions=(16, 16, 16)):
+    """Unsliced output-stationary (reference :220-227)."""
+    R, C = mesh.shape
+    ag_i = estimateAllgather(mesh, (M // R, K // C), 1, precisions[0])
+    ag_w = estimateAllgather(mesh, (K // R, N // C), 0, precisions[1])
+    compute = estimateMatmul(mesh, M // R, N // C, K)
+    return (ag_i, max(compute, ag_w))
+
+
+def GSPMD_LS(mesh, M, N, K, steps=8, precisions=(16, 16, 16)):
+    """Unsliced LHS-stationary (reference :229-237)."""
+    R, C = mesh.shape
+    ag_w = estimateAllgather(mesh, (N // R, K // C), 0, precisions[1])
+    compute = estimateMatmul(mesh, M // R, N, K // C, layout="nt")
+    rs_o = estimateReduceScatter(mesh, (M // R, N // C), 1, precisions[2])
+    return (rs_o, max(ag_w, compute))
+
+
+def GSPMD_RS(mesh, M, N, K, steps=8, precisions=(16, 16, 16)):
+    """Unsliced RHS-stationary (reference :239-247)."""
+    R, C = mesh.shape
+    ag_i = estimateAllgather(mesh, (K // R, M // C), 1, precisions[0])
+    compute = estimateMatmul(mesh, M, N // C, K // R, layout="tn")
+    rs_o = estimateReduceScatter(mesh, (M // R, N // C), 0, precisions[2])
+    return (rs_o, max(ag_i, compute))
+
+
+def MeshFlow_OS(mesh, M, N, K, steps=32, precisions=(16, 16, 16)):
+    """Sliced output-stationary: per slice, gather both operands' slices while the previous slice
+    multiplies (reference :249-258)."""
+    R, C = mesh.shape
+    ag_i = estimateAllgather(mesh, (M // R, K // C // steps), 1, precisions[0])
+    ag_w = estimateAllgather(mesh, (K // R // steps, N // C), 0, precisions[1])
+    compute = estimateMatmul(mesh, M // R, N // C, K // steps)
+    return (max(ag_i, ag_w), max(ag_i, ag_w, compute) * (steps - 1) + compute)
+
+
+def MeshFlow_LS(mesh, M, N, K, steps=32, precisions=(16, 16, 16)):
+    """Sliced LHS-stationary: gather a weight slice, multiply, reduce-scatter the chunk (reference :260-272)."""
+    R, C = mesh.shape
+    ag_w = estimateAllgather(mesh, (N // R // steps, K // C), 0, precisions[1])
+    rs_o = estimateReduceScatter(mesh, (M // R, N // C // steps), 1, precisions[2])
+    compute = estimateMatmul(mesh, M // R, N // steps, K // C, layout="nt")
+    return (ag_w + rs_o, compute + max(ag_w, rs_o, compute) * (steps - 1))
+
+
+def MeshFlow_RS(mesh, M, N, K, steps=32, precisions=(16, 16, 16)):
+    """Sliced RHS-stationary (reference :273-285)."""
+    R, C = mesh.shape
+    ag_i = estimateAllgather(mesh, (K // R, M // C // steps), 1, precisions[0])
+    rs_o = estimateReduceScatter(mesh, (M // R // steps, N // C), 0, precisions[2])
+    compute = estimateMatmul(mesh, M // steps, N // C, K // R, layout="tn")
+    return (ag_i + rs_o, compute + max(ag_i, rs_o, compute) * (steps - 1))
+
+
+def tup2ms(t):
+    return (str(t[0] * 1000) + "ms", str(t[1] * 1000) + "ms", str((t[0] + t[1]) * 1000) + "ms")

@@ -1,0 +1,271 @@
+"""2-D tensor-parallel GEMM: the reference's ``SPMD(mesh, algorithm, blocksize).OS/LS/RS(K)`` surface
+with the mesh emulated on the host and the local contraction running in hand-written gfx950 kernels.
+
+Mirrors reference TensorParallel.py: the unsliced bodies ``Collective_OS/LS/RS`` (:19-32), the sliced
+bodies ``MeshFlow_OS/LS/RS`` (:153-214) and the builder ``SPMD`` (:346-377).  Differences, all forced
+by having one GPU and no tracing compiler:
+
+* the callable returned by ``OS/LS/RS`` takes the GLOBAL operands (torch tensors on the GPU), logically
+  sharded ``P(row, col)``, and returns the GLOBAL result; it runs every mesh device's body in turn;
+* ``.device(i, j)`` runs ONE device's body and returns what that device produces before any
+  cross-device reduction: its output block (OS) or its S fp32 partial chunks (LS / RS);
+* all_gather / psum_scatter are host-side index arithmetic over the list of shards;
+* the local contraction accumulates in fp32 over all slices and rounds once (the reference carries
+  the running sum in the input dtype, :167);
+* the sliced OS body rejects ``K == 1``: the reference adds slice 0 twice in that case (:163,:172);
+  use ``algorithm='collective'`` for the unsliced product;
+* the 'wang' and 'cannon' baselines are not built.
+"""
+from __future__ import annotations
+
+from typing import Callable, List, Sequence
+
+import torch
+
+from . import local_gemm
+from .mesh import Mesh, PartitionSpec as P  # noqa: F401  (re-exported like the reference's imports)
+
+
+def allclose(a, b) -> bool:
+    """The reference's acceptance test (TensorParallel.py:16-17)."""
+    return bool(torch.allclose(torch.as_tensor(a).float().cpu(), torch.as_tensor(b).float().cpu(), atol=1e-2, rtol=1e-2))
+
+
+# ------------------------------------------------------------------------------------------------
+# host-side mesh plumbing
+# ------------------------------------------------------------------------------------------------
+
+def _shards(G: torch.Tensor, R: int, C: int) -> List[List[torch.Tensor]]:
+    """blocks[i][j] = device (i,j)'s shard of a matrix sharded P(row, col) (views, no copies)."""
+    if G.dim() != 2:
+        raise ValueError("operands must be 2-D")
+    if G.shape[0] % R or G.shape[1] % C:
+        raise ValueError(f"matrix {tuple(G.shape)} does not shard evenly over a {R}x{C} mesh")
+    h, w = G.shape[0] // R, G.shape[1] // C
+    return [[G[i * h:(i + 1) * h, j * w:(j + 1) * w] for j in range(C)] for i in range(R)]
+
+
+def _need(v: int, d: int, what: str) -> None:
+    if d <= 0 or v % d:
+        raise ValueError(f"{what} = {v} is not a multiple of {d}")
+
+
+def _slice_cols(block: torch.Tensor, k: int, K: int, B: int) -> torch.Tensor:
+    """Slice k of the column view (rows, cols/(K*B), K, B) -> (rows, cols/K)   (reference :155,157)."""
+    r, c = block.shape
+    _need(c, K * B, "sliced extent")
+    return block.reshape(r, c // (K * B), K, B)[:, :, k, :].reshape(r, c // K)
+
+
+def _slice_rows(block: torch.Tensor, k: int, K: int, B: int) -> torch.Tensor:
+    """Slice k of the row view (rows/(K*B), K, B, cols) -> (rows/K, cols)   (reference :156,158)."""
+    r, c = block.shape
+    _need(r, K * B, "sliced extent")
+    return block.reshape(r // (K * B), K, B, c)[:, k, :, :].reshape(r // K, c)
+
+
+def _gather(parts: Sequence[torch.Tensor], axis: int) -> torch.Tensor:
+    """tiled all_gather as the receiving device sees it: peers' parts concatenated in axis order,
+    materialised contiguous in HBM (what a real all-gather delivers)."""
+    return torch.cat(list(parts), dim=axis).contiguous()
+
+
+# ------------------------------------------------------------------------------------------------
+# per-device bodies.  X, W are the shard grids; (i, j) the device; the return value is what that
+# device holds after its local contractions.
+# ------------------------------------------------------------------------------------------------
+
+def Collective_OS(X, W, i, j, R, C, K, B):
+    """reference TensorParallel.py:19-22: gather X over col, W over row, one contraction."""
+    Xi = _gather([X[i][jj] for jj in range(C)], 1)
+    Wj = _gather([W[ii][j] for ii in range(R)], 0)
+    return local_gemm.gemm_os([Xi], [Wj])
+
+
+def Collective_LS(X, W, i, j, R, C, K, B):
+    """reference :24-27: gather W over row; partial product X_ij @ Wj^T (input of psum_scatter)."""
+    Wj = _gather([W[ii][j] for ii in range(R)], 0)
+    return local_gemm.gemm_ls(X[i][j].contiguous(), [Wj])
+
+
+def Collective_RS(X, W, i, j, R, C, K, B):
+    """reference :29-32: gather X over col; partial product Xi^T @ W_ij (input of psum_scatter)."""
+    Xi = _gather([X[i][jj] for jj in range(C)], 1)
+    return local_gemm.gemm_rs([Xi], W[i][j].contiguous())
+
+
+def MeshFlow_OS(X, W, i, j, R, C, K, B):
+    """reference :153-172: K gathered slice pairs, accumulated into one output block."""
+    if K == 1:
+        raise ValueError("the sliced OS body is undefined for K == 1 (the reference adds slice 0 twice); "
+                         "use algorithm='collective' for the unsliced product")
+    A_slices = [_gather([_slice_cols(X[i][jj], k, K, B) for jj in range(C)], 1) for k in range(K)]
+    B_slices = [_gather([_slice_rows(W[ii][j], k, K, B) for ii in range(R)], 0) for k in range(K)]
+    return local_gemm.gemm_os(A_slices, B_slices)
+
+
+def MeshFlow_LS(X, W, i, j, R, C, K, B):
+    """reference :174-193: K gathered row slices of W; K fp32 partial chunks X_ij @ W_k^T."""
+    W_slices = [_gather([_slice_rows(W[ii][j], k, K, B) for ii in range(R)], 0) for k in range(K)]
+    return local_gemm.gemm_ls(X[i][j].contiguous(), W_slices)
+
+
+def MeshFlow_RS(X, W, i, j, R, C, K, B):
+    """reference :195-214: K gathered column slices of X; K fp32 partial chunks X_k^T @ W_ij."""
+    X_slices = [_gather([_slice_cols(X[i][jj], k, K, B) for jj in range(C)], 1) for k in range(K)]
+    return local_gemm.gemm_rs(X_slices, W[i][j].contiguous())
+
+
+# ------------------------------------------------------------------------------------------------
+# mesh completion: what psum_scatter + the (.., K, B) interleave do with the partial chunks
+# ------------------------------------------------------------------------------------------------
+
+def _finish_ls(chunks_by_col, j, C, K, B, dtype):
+    """psum over the mesh row, keep device column j's blocks, interleave (reference :182-193)."""
+    m, os_ = chunks_by_col[0][0].shape
+    nb = os_ // B                       # B-wide blocks in one gathered slice
+    _need(nb, C, "blocks per slice")
+    out = torch.empty((m, nb // C, K, B), dtype=torch.float32, device=chunks_by_col[0][0].device)
+    for k in range(K):
+        tot = chunks_by_col[0][k].clone()
+        for jj in range(1, C):
+            tot += chunks_by_col[jj][k]
+        out[:, :, k, :] = tot.reshape(m, nb, B)[:, j * (nb // C):(j + 1) * (nb // C), :]
+    return out.reshape(m, -1).to(dtype)
+
+
+def _finish_rs(chunks_by_row, i, R, K, B, dtype):
+    """psum over the mesh column, keep device row i's blocks, interleave (reference :204-214)."""
+    ns, n = chunks_by_row[0][0].shape
+    nb = ns // B
+    _need(nb, R, "blocks per slice")
+    out = torch.empty((nb // R, K, B, n), dtype=torch.float32, device=chunks_by_row[0][0].device)
+    for k in range(K):
+        tot = chunks_by_row[0][k].clone()
+        for ii in range(1, R):
+            tot += chunks_by_row[ii][k]
+        out[:, k, :, :] = tot.reshape(nb, B, n)[i * (nb // R):(i + 1) * (nb // R), :, :]
+    return out.reshape(-1, n).to(dtype)
+
+
+class ShardedMatmul:
+    """What ``SPMD.OS/LS/RS(K)`` returns: ``f(X, W) -> Y`` on global operands, plus ``f.device(i, j)``."""
+
+    def __init__(self, dataflow: str, body: Callable, mesh: Mesh, K: int, B: int, sliced: bool):
+        self.dataflow, self.body, self.mesh, self.K, self.B, self.sliced = dataflow, body, mesh, int(K), int(B), sliced
+        self.R, self.C = mesh.shape
+
+    # shape rules implied by the reference's reshapes (:155-156,177-179,198-200)
+    def _validate(self, X: torch.Tensor, W: torch.Tensor) -> None:
+        R, C = self.R, self.C
+        S = self.K if self.sliced else 1
+        B = self.B if self.sliced else 1
+        if S < 1:
+            raise ValueError(f"slice count must be >= 1, got {S}")
+        for t, name in ((X, "X"), (W, "W")):
+            if not isinstance(t, torch.Tensor) or t.dim() != 2:
+                raise ValueError(f"{name} must be a 2-D torch tensor")
+        if X.dtype != W.dtype:
+            raise ValueError("X and W must share a dtype")
+        if self.dataflow == "os":
+            if X.shape[1] != W.shape[0]:
+                raise ValueError(f"os: cannot contract {tuple(X.shape)} @ {tuple(W.shape)}")
+            _need(X.shape[0], R, "rows of X"); _need(W.shape[1], C, "cols of W")
+            _need(X.shape[1], C * S * B, "cols of X"); _need(W.shape[0], R * S * B, "rows of W")
+        elif self.dataflow == "ls":
+            if X.shape[1] != W.shape[1]:
+                raise ValueError(f"ls: cannot contract {tuple(X.shape)} @ {tuple(W.shape)}^T")
+            _need(X.shape[0], R, "rows of X"); _need(X.shape[1], C, "cols of X")
+            _need(W.shape[0], R * S * B, "rows of W"); _need(W.shape[0], C * S * B, "rows of W")
+        else:
+            if X.shape[0] != W.shape[0]:
+                raise ValueError(f"rs: cannot contract {tuple(X.shape)}^T @ {tuple(W.shape)}")
+            _need(X.shape[0], R, "rows of X"); _need(W.shape[1], C, "cols of W")
+            _need(X.shape[1], C * S * B, "cols of X"); _need(X.shape[1], R * S * B, "cols of X")
+        for t, name in ((X, "X"), (W, "W")):
+            if not t.is_cuda:
+                raise local_gemm._lib.MeshSliceError(f"{name} must live on the GPU: there is no CPU path")
+
+    def device(self, i: int, j: int) -> Callable:
+        """Body of mesh device (i, j): returns its output block (OS) or its fp32 partial chunks."""
+        if not (0 <= i < self.R and 0 <= j < self.C):
+            raise ValueError(f"device ({i},{j}) is outside the {self.R}x{self.C} mesh")
+
+        def run(X, W):
+            self._validate(X, W)
+            return self.body(_shards(X, self.R, self.C), _shards(W, self.R, self.C), i, j, self.R, self.C, self.K, self.B)
+        return run
+
+    def __call__(self, X: torch.Tensor, W: torch.Tensor) -> torch.Tensor:
+        self._validate(X, W)
+        R, C = self.R, self.C
+        K = self.K if self.sliced else 1
+        B = self.B if self.sliced else 1
+        Xs, Ws = _shards(X, R, C), _shards(W, R, C)
+        run = lambda i, j: self.body(Xs, Ws, i, j, R, C, self.K, self.B)
+        if self.dataflow == "os":
+            return torch.cat([torch.cat([run(i, j) for j in range(C)], dim=1) for i in range(R)], dim=0)
+        if self.dataflow == "ls":
+            rows = []
+            for i in range(R):
+                chunks = [run(i, j) for j in range(C)]
+                if not self.sliced:  # one chunk: tiled scatter of contiguous column blocks
+                    tot = sum(c[0] for c in chunks)
+                    rows.append(tot.to(X.dtype))
+                else:
+                    rows.append(torch.cat([_finish_ls(chunks, j, C, K, B, X.dtype) for j in range(C)], dim=1))
+            return torch.cat(rows, dim=0)
+        cols = []
+        for j in range(C):
+            chunks = [run(i, j) for i in range(R)]
+            if not self.sliced:
+                cols.append(sum(c[0] for c in chunks).to(X.dtype))
+            else:
+                cols.append(torch.cat([_finish_rs(chunks, i, R, K, B, X.dtype) for i in range(R)], dim=0))
+        return torch.cat(cols, dim=1)
+
+
+class SPMD:
+    """reference TensorParallel.py:346-377.  ``jit`` is accepted and ignored: kernels are ahead-of-time
+    compiled."""
+
+    def __init__(self, mesh: Mesh, algorithm: str = "collective", blocksize: int = 8, jit: bool = True):
+        self.mesh = mesh
+        self.rowaxis = mesh.axis_names[0]
+        self.colaxis = mesh.axis_names[1]
+        self.spec = P(self.rowaxis, self.colaxis)
+        self.blocksize = blocksize
+        self.jit = jit
+        self.algorithm = algorithm
+        if algorithm == "collective":
+            self.funcs = {"os": Collective_OS, "ls": Collective_LS, "rs": Collective_RS}
+            self.sliced = False
+        elif algorithm in ("wang", "cannon"):
+            raise NotImplementedError(
+                f"algorithm {algorithm!r} (a comparison baseline of the reference) is not part of this build; "
+                "use 'collective' or 'meshflow'")
+        else:  # like the reference, any other name selects the sliced MeshFlow bodies
+            self.funcs = {"os": MeshFlow_OS, "ls": MeshFlow_LS, "rs": MeshFlow_RS}
+            self.sliced = True
+
+    def _build(self, which: str, K: int) -> ShardedMatmul:
+        if int(K) < 1:
+            raise ValueError(f"slice count K must be >= 1, got {K}")
+        return ShardedMatmul(which, self.funcs[which], self.mesh, K, self.blocksize, self.sliced)
+
+    def OS(self, K: int = 8) -> ShardedMatmul:
+        return self._build("os", K)
+
+    def LS(self, K: int = 8) -> ShardedMatmul:
+        return self._build("ls", K)
+
+    def RS(self, K: int = 8) -> ShardedMatmul:
+        return self._build("rs", K)
+
+
+def createMultihostMatrix(mesh: Mesh, sharding, global_shape, dtype=torch.bfloat16, seed: int = 0, device="cuda"):
+    """reference :419-423: a random N(0,1) matrix of ``global_shape`` sharded over the mesh.  The
+    reference seeds JAX's generator with the process index; this build has one process and uses
+    torch's generator with ``seed`` (the sample streams differ; nothing depends on them)."""
+    g = torch.Generator(device="cpu").manual_seed(int(seed))
+    return torch.randn(tuple(global_shape), generator=g, dtype=torch.float32).to(dtype).to(device)

@@ -1,0 +1,280 @@
+"""Parity of the HIP path against the oracle, through the C ABI, on the GPU.
+
+Tolerances (rel-Frobenius error ||C - C_ref||_F / ||C_ref||_F against the float64 oracle evaluated on
+the dtype-rounded inputs): 1e-5 for fp32 in / fp32 out, 1e-2 for bf16 in / fp32 accumulate.
+"""
+import ctypes
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import meshslice_oracle as orc
+import meshslice_amd as ms
+from meshslice_amd import _lib
+from meshslice_amd import TensorParallel as TP
+from meshslice_amd.ShardedLayers import ShardedFFLayer
+from meshslice_amd.mesh import Mesh, create_device_mesh
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOL_F32 = 1e-5
+TOL_BF16 = 1e-2
+
+
+def dev(a, dtype=torch.float32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda").to(dtype)
+
+
+def host(t):
+    return t.detach().float().cpu().numpy().astype(np.float64)
+
+
+@pytest.fixture(autouse=True)
+def _default_variant():
+    _lib.load().ms_set_variant(0)
+    yield
+    _lib.load().ms_set_variant(0)
+    torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------ BASELINE config 1 (fp32 plumbing check)
+def test_config1_fp32_os_device00_matches_oracle():
+    rng = np.random.default_rng(0)
+    A = rng.standard_normal((1024, 1024)).astype(np.float32)
+    B = rng.standard_normal((1024, 1024)).astype(np.float32)
+    R = C = 2; S = 4; blk = 8
+    As, Bs = orc.device_operands_os(A, B, R, C, 0, 0, S, blk)
+    assert As[0].shape == (512, 256) and Bs[0].shape == (256, 512)
+    got = ms.gemm_os([dev(a) for a in As], [dev(b) for b in Bs])
+    want = orc.oracle_os_block(As, Bs)
+    assert np.array_equal(want, A[:512].astype(np.float64) @ B[:, :512].astype(np.float64)) or \
+        orc.rel_frobenius(want, A[:512].astype(np.float64) @ B[:, :512].astype(np.float64)) < 1e-14
+    assert orc.rel_frobenius(host(got), want) <= TOL_F32
+    # the same block through the reference-shaped API
+    mesh = Mesh(create_device_mesh((2, 2)), ("row", "col"))
+    blk00 = TP.SPMD(mesh, "meshflow").OS(4).device(0, 0)(dev(A), dev(B))
+    assert torch.equal(blk00, got)
+
+
+# ------------------------------------------------------------------ notebook walkthrough (known answers)
+@pytest.fixture(scope="module")
+def nb():
+    d = orc.notebook_inputs(np.float32)
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "notebook_blocks.json")))
+    return d, g
+
+
+@pytest.mark.parametrize("alg", ["collective", "meshflow"])
+@pytest.mark.parametrize("flow", ["os", "ls", "rs"])
+def test_notebook_whole_mesh_matches_golden_and_reference_allclose(nb, alg, flow):
+    d, g = nb
+    mesh = Mesh(create_device_mesh(d["mesh"]), ("row", "col"))
+    X, W = {"os": (d["X"], d["W"]), "ls": (d["dY"], d["W"]), "rs": (d["X"], d["dY"])}[flow]
+    f = getattr(TP.SPMD(mesh, alg), flow.upper())()         # default K=8, blocksize=8 as in the notebook
+    Y = host(f(dev(X), dev(W)))
+    want = orc.dense(flow, X, W)
+    assert orc.allclose(Y, want)                              # the reference's own criterion
+    assert orc.rel_frobenius(Y, want) <= TOL_F32
+    R, C = d["mesh"]
+    for key, st in g[flow].items():
+        i, j = map(int, key.split(","))
+        blk = orc.shard(Y, R, C, i, j)
+        assert blk.sum() == pytest.approx(st["sum"], rel=1e-5)
+        assert np.allclose([blk[0, 0], blk[0, -1], blk[-1, 0], blk[-1, -1]], st["corners"], rtol=2e-5, atol=0)
+
+
+def test_selfcheck_chain_on_one_device():
+    """TensorParallel.py:433-457 on the 4x4 mesh: Yo=OS(X,W); LS(Yo,W); RS(X,Yo); device (2,1)."""
+    d = orc.selfcheck_inputs(np.float32)
+    R, C = d["mesh"]; S, B = d["K"], d["blocksize"]
+    mesh = Mesh(create_device_mesh((R, C)), ("x", "y"))
+    alg = TP.SPMD(mesh, "meshflow")
+    X, W = dev(d["X"]), dev(d["W"])
+    i, j = 2, 1
+    blk = alg.OS().device(i, j)(X, W)
+    want = orc.oracle_os_block(*orc.device_operands_os(d["X"], d["W"], R, C, i, j, S, B))
+    assert orc.rel_frobenius(host(blk), want) <= TOL_F32
+    Yo = (d["X"].astype(np.float64) @ d["W"].astype(np.float64)).astype(np.float32)
+    chunks = alg.LS().device(i, j)(dev(Yo), W)
+    want = orc.oracle_ls_chunks(*orc.device_operands_ls(Yo, d["W"], R, C, i, j, S, B))
+    assert max(orc.rel_frobenius(host(c), w) for c, w in zip(chunks, want)) <= TOL_F32
+    chunks = alg.RS().device(i, j)(X, dev(Yo))
+    want = orc.oracle_rs_chunks(*orc.device_operands_rs(d["X"], Yo, R, C, i, j, S, B))
+    assert max(orc.rel_frobenius(host(c), w) for c, w in zip(chunks, want)) <= TOL_F32
+
+
+# ------------------------------------------------------------------ seeded random cases, every kernel variant
+SHAPES = [  # (m, n, k_or_slice, S)
+    (512, 512, 256, 4),
+    (256, 256, 64, 1),       # a single K step
+    (256, 256, 192, 1),      # odd number of K steps
+    (1000, 776, 328, 3),     # ragged in every dimension, K tail of 8
+    (264, 520, 72, 2),       # K tail after one full step, per slice
+    (8, 8, 8, 1),            # smallest admissible problem
+    (40, 4096, 136, 16),     # wide and thin, many slices
+]
+
+
+def _rand_case(flow, m, n, k, S, seed, dtype):
+    rng = np.random.default_rng(seed)
+    rnd = (lambda s, sc=1.0: orc.bf16_round(rng.standard_normal(s).astype(np.float32) * sc)) if dtype == torch.bfloat16 \
+        else (lambda s, sc=1.0: rng.standard_normal(s).astype(np.float32) * np.float32(sc))
+    if flow == "os":
+        return [rnd((m, k)) for _ in range(S)], [rnd((k, n), 0.05) for _ in range(S)]
+    if flow == "ls":
+        return rnd((m, k)), [rnd((n, k), 0.05) for _ in range(S)]
+    return [rnd((k, m)) for _ in range(S)], rnd((k, n), 0.05)
+
+
+def _run_and_compare(flow, ops, dtype, tol, out_dtype=None):
+    if flow == "os":
+        A, B = ops
+        got = ms.gemm_os([dev(a, dtype) for a in A], [dev(b, dtype) for b in B], out_dtype=out_dtype)
+        err = orc.rel_frobenius(host(got), orc.oracle_os_block(A, B))
+    elif flow == "ls":
+        A, W = ops
+        got = ms.gemm_ls(dev(A, dtype), [dev(w, dtype) for w in W])
+        err = max(orc.rel_frobenius(host(g), w) for g, w in zip(got, orc.oracle_ls_chunks(A, W)))
+    else:
+        X, W = ops
+        got = ms.gemm_rs([dev(x, dtype) for x in X], dev(W, dtype))
+        err = max(orc.rel_frobenius(host(g), w) for g, w in zip(got, orc.oracle_rs_chunks(X, W)))
+    assert err <= tol, f"{flow}: rel-Frobenius {err:.3e} > {tol}"
+    return err
+
+
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("flow", ["os", "ls", "rs"])
+def test_bf16_random_cases_all_variants(flow, variant):
+    _lib.check(_lib.load().ms_set_variant(variant))
+    for idx, (m, n, k, S) in enumerate(SHAPES):
+        ops = _rand_case(flow, m, n, k, S, seed=100 * idx + variant, dtype=torch.bfloat16)
+        _run_and_compare(flow, ops, torch.bfloat16, TOL_BF16)
+        if flow != "os":
+            continue
+        # fp32 output of the same accumulators is far inside the bf16 tolerance
+        err = _run_and_compare(flow, ops, torch.bfloat16, TOL_BF16, out_dtype=torch.float32)
+        assert err < 1e-5
+
+
+@pytest.mark.parametrize("flow", ["os", "ls", "rs"])
+def test_fp32_random_cases(flow):
+    for idx, (m, n, k, S) in enumerate(SHAPES + [(200, 136, 100, 3), (68, 60, 20, 2)]):
+        ops = _rand_case(flow, m, n, k, S, seed=7 + idx, dtype=torch.float32)
+        _run_and_compare(flow, ops, torch.float32, TOL_F32)
+
+
+def test_bf16_output_is_one_rounding_of_the_fp32_accumulator():
+    """OS accumulates all slices in fp32 and rounds once: the bf16 result equals the round-to-nearest-even
+    of the fp32-output result of the same call, bit for bit."""
+    A, B = _rand_case("os", 512, 768, 256, 4, seed=3, dtype=torch.bfloat16)
+    a = [dev(x, torch.bfloat16) for x in A]; b = [dev(x, torch.bfloat16) for x in B]
+    c32 = ms.gemm_os(a, b, out_dtype=torch.float32)
+    c16 = ms.gemm_os(a, b, out_dtype=torch.bfloat16)
+    want = orc.bf16_bits(c32.cpu().numpy())
+    got = c16.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_strided_operands_and_outputs():
+    """Leading dimensions larger than the row length (slices that are views of a bigger buffer)."""
+    rng = np.random.default_rng(5)
+    m, n, k, S = 300, 264, 128, 2
+    bigA = orc.bf16_round(rng.standard_normal((m, S * k + 16)).astype(np.float32))
+    bigB = orc.bf16_round(rng.standard_normal((S * k, n + 40)).astype(np.float32) * 0.05)
+    dA, dB = dev(bigA, torch.bfloat16), dev(bigB, torch.bfloat16)
+    A = [dA[:, s * k:(s + 1) * k] for s in range(S)]
+    B = [dB[s * k:(s + 1) * k, :n] for s in range(S)]
+    out = torch.zeros((m, n + 24), dtype=torch.bfloat16, device="cuda")
+    ms.gemm_os(A, B, out=out[:, :n])
+    want = orc.oracle_os_block([bigA[:, s * k:(s + 1) * k] for s in range(S)], [bigB[s * k:(s + 1) * k, :n] for s in range(S)])
+    assert orc.rel_frobenius(host(out[:, :n]), want) <= TOL_BF16
+    assert float(out[:, n:].abs().max()) == 0.0            # nothing written outside the block
+
+
+# ------------------------------------------------------------------ whole-mesh API on random bf16 data
+@pytest.mark.parametrize("R,C,K", [(2, 2, 2), (4, 2, 4), (2, 4, 2)])
+@pytest.mark.parametrize("flow", ["os", "ls", "rs"])
+def test_meshflow_equals_collective_equals_dense(flow, R, C, K):
+    rng = np.random.default_rng(R * 10 + C + K)
+    u = R * C * K * 8
+    shp = {"os": ((4 * R * 8, u), (u, 2 * u)), "ls": ((4 * R * 8, 2 * C * 16), (u, 2 * C * 16)),
+           "rs": ((4 * R * 8, u), (4 * R * 8, 3 * C * 8))}[flow]
+    X = orc.bf16_round(rng.standard_normal(shp[0]).astype(np.float32))
+    W = orc.bf16_round(rng.standard_normal(shp[1]).astype(np.float32) * 0.1)
+    mesh = Mesh(create_device_mesh((R, C)), ("row", "col"))
+    dX, dW = dev(X, torch.bfloat16), dev(W, torch.bfloat16)
+    want = orc.dense(flow, X, W)
+    y_c = getattr(TP.SPMD(mesh, "collective"), flow.upper())(K)(dX, dW)
+    y_m = getattr(TP.SPMD(mesh, "meshflow"), flow.upper())(K)(dX, dW)
+    assert y_c.dtype == torch.bfloat16 and y_m.dtype == torch.bfloat16 and tuple(y_m.shape) == want.shape
+    assert orc.rel_frobenius(host(y_c), want) <= TOL_BF16
+    assert orc.rel_frobenius(host(y_m), want) <= TOL_BF16
+    assert TP.allclose(y_m, y_c)
+    # the sliced result also matches the literal whole-mesh emulation of the reference body
+    lit = orc.literal_meshflow(flow, X.astype(np.float64), W.astype(np.float64), R, C, K, 8)
+    assert orc.rel_frobenius(host(y_m), lit) <= TOL_BF16
+
+
+@pytest.mark.parametrize("dataflow", ["os", "ls", "rs"])
+def test_sharded_ff_layer_forward_and_vjp(dataflow):
+    """reference ShardedLayers.py:41-81: (fwd, dx, dw) = (OS,LS,RS) / (LS,OS,RS) / (RS,LS,OS)."""
+    mesh = Mesh(create_device_mesh((2, 2)), ("row", "col"))
+    tokens, in_dim, out_dim, ks = 128, 64, 96, 2
+    layer = ShardedFFLayer(mesh, "meshflow", dataflow, ks, in_dim, out_dim, seed=4)
+    assert tuple(layer.weight.shape) == ((out_dim, in_dim) if dataflow == "ls" else (in_dim, out_dim))
+    assert layer.weight.dtype == torch.bfloat16
+    g = torch.Generator().manual_seed(9)
+    xs = (in_dim, tokens) if dataflow == "rs" else (tokens, in_dim)
+    x = torch.randn(xs, generator=g).to(torch.bfloat16).cuda().requires_grad_(True)
+    w = layer.weight.clone().requires_grad_(True)
+    y = layer.forward(x, w)
+    xr = x.detach().double().requires_grad_(True); wr = w.detach().double().requires_grad_(True)
+    yr = {"os": lambda: xr @ wr, "ls": lambda: xr @ wr.t(), "rs": lambda: xr.t() @ wr}[dataflow]()
+    assert orc.rel_frobenius(host(y), yr.detach().cpu().numpy()) <= TOL_BF16
+    dy = torch.randn(tuple(y.shape), generator=g).to(torch.bfloat16).cuda()
+    y.backward(dy)
+    yr.backward(dy.double())
+    assert orc.rel_frobenius(host(x.grad), xr.grad.cpu().numpy()) <= TOL_BF16
+    assert orc.rel_frobenius(host(w.grad), wr.grad.cpu().numpy()) <= TOL_BF16
+
+
+# ------------------------------------------------------------------ error behaviour through the C ABI
+def test_c_abi_rejects_bad_arguments():
+    lib = _lib.load()
+    a = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
+    c = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
+    pa, _k1 = _lib.ptr_array([a.data_ptr()]); pb, _k2 = _lib.ptr_array([a.data_ptr()])
+    vp = ctypes.c_void_p
+    call = lambda **kw: lib.ms_gemm_os(kw.get("pa", pa), kw.get("pb", pb), kw.get("S", 1), kw.get("m", 64), kw.get("n", 64),
+                                       kw.get("k", 64), kw.get("lda", 64), kw.get("ldb", 64), vp(kw.get("c", c.data_ptr())),
+                                       kw.get("ldc", 64), kw.get("idt", 1), kw.get("odt", 1), None)
+    assert call() == _lib.MS_OK
+    assert call(S=0) == _lib.MS_ERR_ARG and "S = 0" in _lib.last_error()
+    assert call(S=65) == _lib.MS_ERR_ARG
+    assert call(m=0) == _lib.MS_ERR_ARG
+    assert call(k=60) == _lib.MS_ERR_ARG           # contiguous extent not a multiple of 8
+    assert call(lda=32) == _lib.MS_ERR_ARG         # leading dimension smaller than the row
+    assert call(c=c.data_ptr() + 2) == _lib.MS_ERR_ARG
+    assert call(c=0) == _lib.MS_ERR_ARG
+    assert call(idt=7) == _lib.MS_ERR_UNSUPPORTED
+    null, _k3 = _lib.ptr_array([0])
+    assert call(pa=null) == _lib.MS_ERR_ARG
+    assert lib.ms_set_variant(99) == _lib.MS_ERR_ARG
+    with pytest.raises(ValueError):
+        ms.gemm_os([a], [torch.zeros((32, 64), dtype=torch.bfloat16, device="cuda")])
+    with pytest.raises(ValueError):
+        _lib.check(call(S=0))
+    torch.cuda.synchronize()
+
+
+def test_query_reports_the_device():
+    lib = _lib.load()
+    assert lib.ms_query(_lib.MS_QUERY_IS_GFX950) == 1
+    assert lib.ms_query(_lib.MS_QUERY_CU_COUNT) == torch.cuda.get_device_properties(0).multi_processor_count
+    assert lib.ms_query(_lib.MS_QUERY_LDS_BYTES) >= 160 * 1024
+    assert lib.ms_query(1234) == -1

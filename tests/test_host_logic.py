@@ -1,0 +1,243 @@
+"""Host-side logic that needs no GPU: the C ABI loads and exports what the header declares, the mesh
+plumbing of TensorParallel.py agrees with the oracle's closed forms, the cost model's formulas match
+hand-computed values, and the golden fixtures agree with the oracle."""
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import meshslice_oracle as orc
+import meshslice_amd
+from meshslice_amd import _lib, CostModel, Autotuner
+from meshslice_amd import TensorParallel as TP
+from meshslice_amd.mesh import Mesh, create_device_mesh
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---------------------------------------------------------------- C ABI
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "meshslice_hip.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(ms_[a-z_0-9]+)\s*\(", header))
+    assert {"ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_version", "ms_last_error", "ms_query"} <= declared
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert set(_lib.EXPORTS) == declared
+    assert lib.ms_version() >= 100
+    assert lib.ms_query(_lib.MS_QUERY_MAX_SLICES) == 64
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libmeshslice_hip.so")
+    with pytest.raises(_lib.MeshSliceError, match="no CPU fallback"):
+        _lib.load()
+
+
+def test_cpu_tensors_are_rejected_not_computed():
+    a = torch.zeros(8, 8); b = torch.zeros(8, 8)
+    with pytest.raises(_lib.MeshSliceError):
+        meshslice_amd.gemm_os([a], [b])
+    mesh = Mesh(create_device_mesh((2, 2)), ("row", "col"))
+    with pytest.raises(_lib.MeshSliceError):
+        TP.SPMD(mesh, "collective").OS()(torch.zeros(16, 16), torch.zeros(16, 16))
+
+
+# ---------------------------------------------------------------- mesh plumbing vs oracle
+@pytest.mark.parametrize("R,C,K,B", [(2, 2, 2, 2), (4, 2, 8, 8), (2, 4, 4, 8)])
+def test_slice_and_gather_match_closed_form(R, C, K, B):
+    L = R * C * K * B * 2
+    G = torch.arange(24 * L, dtype=torch.float32).reshape(24, L)
+    Xs = TP._shards(G, 4, C)
+    for k in range(K):
+        got = TP._gather([TP._slice_cols(Xs[1][jj], k, K, B) for jj in range(C)], 1)
+        want = G[6:12][:, torch.from_numpy(orc.sel(L, K, B, k))]
+        assert torch.equal(got, want)
+    Gt = G.t().contiguous()
+    Ws = TP._shards(Gt, R, 4)
+    for k in range(K):
+        got = TP._gather([TP._slice_rows(Ws[ii][2], k, K, B) for ii in range(R)], 0)
+        want = Gt[:, 12:18][torch.from_numpy(orc.sel(L, K, B, k)), :]
+        assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("R,C,S,B", [(2, 2, 2, 2), (4, 2, 4, 8), (2, 4, 2, 8)])
+def test_chunk_assembly_matches_oracle(R, C, S, B):
+    rng = np.random.default_rng(11)
+    O = R * C * S * B * 2
+    m = 6
+    chunks = [[rng.integers(-5, 6, (m, O // S)).astype(np.float32) for _ in range(S)] for _ in range(C)]
+    tch = [[torch.from_numpy(c) for c in row] for row in chunks]
+    for j in range(C):
+        got = TP._finish_ls(tch, j, C, S, B, torch.float32).numpy()
+        assert np.array_equal(got, orc.assemble_ls(chunks, R, C, j, S, B))
+    n = 5
+    chunks = [[rng.integers(-5, 6, (O // S, n)).astype(np.float32) for _ in range(S)] for _ in range(R)]
+    tch = [[torch.from_numpy(c) for c in row] for row in chunks]
+    for i in range(R):
+        got = TP._finish_rs(tch, i, R, S, B, torch.float32).numpy()
+        assert np.array_equal(got, orc.assemble_rs(chunks, R, C, i, S, B))
+
+
+def test_spmd_surface_and_shape_errors():
+    mesh = Mesh(create_device_mesh((4, 2)), ("row", "col"))
+    assert mesh.axis_names == ("row", "col") and mesh.devices.shape == (4, 2)
+    s = TP.SPMD(mesh, "meshflow")
+    assert s.blocksize == 8 and s.rowaxis == "row" and s.colaxis == "col"
+    for name in ("systolic", "noff", "meshflow"):      # any other name selects the sliced bodies
+        assert TP.SPMD(mesh, name).funcs["os"] is TP.MeshFlow_OS
+    assert TP.SPMD(mesh, "collective").funcs["ls"] is TP.Collective_LS
+    with pytest.raises(NotImplementedError):
+        TP.SPMD(mesh, "cannon")
+    f = s.OS()                                          # default K = 8
+    assert f.K == 8
+    with pytest.raises(ValueError):                     # 256/2 = 128 per shard, needs multiple of 8*8
+        f(torch.zeros(512, 96), torch.zeros(96, 1024))
+    with pytest.raises(ValueError):
+        s.LS(0)
+    with pytest.raises(ValueError):
+        f.device(4, 0)
+    with pytest.raises(ValueError, match="K == 1"):
+        TP.MeshFlow_OS(None, None, 0, 0, 4, 2, 1, 8)
+
+
+# ---------------------------------------------------------------- cost model
+def _mesh(shape):
+    return Autotuner.default_mesh(shape)
+
+
+def test_ring_collective_estimates_by_hand():
+    m = _mesh((4, 4))
+    # all-gather of a [1024, 96] bf16 shard along dim 1: 3 steps of 196608 B at 79.751 GB/s + 3*5us + 13us
+    want = 13e-6 + 3 * (1024 * 96 * 2 / 79.751e9) + 3 * 5e-6
+    assert CostModel.estimateAllgather(m, (1024, 96), 1, 16) == pytest.approx(want, rel=1e-12)
+    want = 26e-6 + 3 * (512 * 64 * 2 / 37.506e9) + 3 * 5e-6
+    assert CostModel.estimateReduceScatter(m, (512, 64), 0, 16) == pytest.approx(want, rel=1e-12)
+    sub = _mesh(((2, 2), 4))
+    assert sub.shape == (4, 4) and sub.meshdim == 0 and sub.submesh == (2, 2)
+    half = (512 * 64 * 2) // 2
+    bw = 27.472e9
+    want = 13e-6 + max(half / bw + half * 2 / bw, half / bw + half * 2 / bw) + 5e-6 * 2
+    assert CostModel.estimateAllgather(sub, (512, 64), 0, 16) == pytest.approx(want, rel=1e-12)
+
+
+def test_meshflow_models_use_per_slice_shapes_and_compose_by_hand():
+    calls = []
+    term = CostModel.ComputeTerm()
+
+    class Spy(CostModel.ComputeTerm):
+        def seconds(self, M, N, K, layout):
+            calls.append((M, N, K, layout))
+            return 1e-4
+    CostModel.use_compute_term(Spy())
+    try:
+        m = _mesh((4, 4))
+        M, N, K, S = 16384, 49152, 12288, 4
+        pro, steady = CostModel.MeshFlow_OS(m, M, N, K, S)
+        assert calls[-1] == (4096, 12288, 3072, "nn")
+        ag_i = CostModel.estimateAllgather(m, (4096, 768), 1, 16)
+        ag_w = CostModel.estimateAllgather(m, (768, 12288), 0, 16)
+        assert pro == pytest.approx(max(ag_i, ag_w))
+        assert steady == pytest.approx(max(ag_i, ag_w, 1e-4) * 3 + 1e-4)
+        pro, steady = CostModel.MeshFlow_LS(m, 16384, 12288, 49152, 8)
+        assert calls[-1] == (4096, 1536, 12288, "nt")
+        ag = CostModel.estimateAllgather(m, (384, 12288), 0, 16)
+        rs = CostModel.estimateReduceScatter(m, (4096, 384), 1, 16)
+        assert pro == pytest.approx(ag + rs) and steady == pytest.approx(1e-4 + max(ag, rs, 1e-4) * 7)
+        pro, steady = CostModel.MeshFlow_RS(m, 12288, 49152, 16384, 4)
+        assert calls[-1] == (3072, 12288, 4096, "tn")
+        CostModel.GSPMD_OS(m, M, N, K)
+        assert calls[-1] == (4096, 12288, 12288, "nn")
+        CostModel.GSPMD_LS(m, 16384, 12288, 49152)
+        assert calls[-1] == (4096, 12288, 12288, "nt")
+        CostModel.GSPMD_RS(m, 12288, 49152, 16384)
+        assert calls[-1] == (12288, 12288, 4096, "tn")
+    finally:
+        CostModel.use_compute_term(None)
+    assert term.table == {}
+
+
+def test_compute_term_fit_recovers_a_planted_model():
+    peak = CostModel.BF16_PEAK_FLOPS
+    t0, eta = 7e-6, 0.6
+    shapes = [(4096, 12288, 768), (4096, 12288, 3072), (2048, 6144, 1536), (8192, 6144, 12288)]
+    samples = [(m, n, k, "nn", t0 + 2.0 * m * n * k / (eta * peak)) for m, n, k in shapes]
+    ct = CostModel.fit_compute_term(samples)
+    assert ct.t0["nn"] == pytest.approx(t0, rel=1e-6) and ct.eta["nn"] == pytest.approx(eta, rel=1e-6)
+    assert ct.seconds(4096, 12288, 768, "nn") == samples[0][4]           # table hit
+    assert ct.seconds(1024, 1024, 1024, "nn") == pytest.approx(t0 + 2.0 * 1024**3 / (eta * peak))
+    back = CostModel.ComputeTerm.from_dict(json.loads(json.dumps(ct.to_dict())))
+    assert back.seconds(4096, 12288, 3072, "nn") == samples[1][4]
+    with pytest.raises(KeyError):
+        ct.seconds(8, 8, 8, "tn")
+
+
+def test_estimate_matmul_without_gpu_or_term_raises():
+    CostModel.use_compute_term(None)
+    if torch.cuda.is_available():
+        pytest.skip("GPU present")
+    with pytest.raises(_lib.MeshSliceError):
+        CostModel.estimateMatmul(None, 256, 256, 256)
+    with pytest.raises(ValueError):
+        CostModel.estimateMatmul(None, 8, 8, 8, layout="tt")
+
+
+def test_possible_k_and_layer_passes():
+    # reference Autotuner.py:242-273 on the GPT-3 layer: 12288 / lcm(4,4) / 8 = 384 = 48*8
+    assert Autotuner.possibleK(16384, 12288, 49152, (4, 4), "os") == [3, 4, 6, 8, 12, 16, 24]
+    assert Autotuner.possibleK(16384, 12288, 49152, (8, 8), "os") == [3, 4, 6, 8, 12, 16, 24]  # 192
+    assert Autotuner.possibleK(16384, 49152, 12288, (2, 8), "ls") == [3, 4, 6, 8, 12, 16, 24]
+    assert Autotuner.possibleK(4096, 1280, 5120, (4, 4), "os") == [4, 5, 8, 10, 20]            # 40
+    assert Autotuner.possibleK(7 * 2 * 8, 8, 8, (2, 2), "rs") == [7]                                 # fallback
+    assert Autotuner.pick_dataflow(16384, 12288, 49152) == "os"
+    assert Autotuner.pick_dataflow(16384, 49152, 12288) == "ls"
+    assert Autotuner.pick_dataflow(64, 4096, 4096) == "rs"
+    f = Autotuner.FFLayerModel(16384, 12288, 49152, "os")
+    assert f.passes() == [("os", 16384, 49152, 12288), ("ls", 16384, 12288, 49152), ("rs", 12288, 49152, 16384)]
+    shapes = Autotuner.per_slice_shapes(16384, 12288, 49152, "os", (4, 4), 4)
+    assert shapes == [("fwd", 4096, 12288, 3072, "nn"), ("bwd_data", 4096, 3072, 12288, "nt"),
+                      ("bwd_weight", 3072, 12288, 4096, "tn")]
+    ls = Autotuner.per_slice_shapes(16384, 49152, 12288, "ls", (4, 4), 8, passes=("fwd",))
+    assert ls == [("fwd", 4096, 1536, 12288, "nt")]
+
+
+def test_emulate_ff_time_scans_slice_counts():
+    class Flat(CostModel.ComputeTerm):
+        def seconds(self, M, N, K, layout):
+            return 2.0 * M * N * K / 1.5e15 + 5e-6      # fixed launch cost favours fewer slices
+    CostModel.use_compute_term(Flat())
+    try:
+        layers = [(16384, 12288, 49152, "os"), (16384, 49152, 12288, "ls")]
+        total, best = Autotuner.emulateFFTime(layers, (4, 4), sweep=True)
+        by_hand = []
+        for (B, I, O, df) in layers:
+            model = Autotuner.FFLayerModel(B, I, O, df)
+            times = {k: model.emulate(Autotuner.default_mesh((4, 4)), k) for k in Autotuner.possibleK(B, I, O, (4, 4), df)}
+            by_hand.append(min(times, key=times.get))
+            assert times[by_hand[-1]] <= min(times.values())
+        assert best == by_hand
+        t2, b2 = Autotuner.emulateFFTime(layers, (4, 4), sweep=False)
+        assert t2 >= total
+    finally:
+        CostModel.use_compute_term(None)
+
+
+# ---------------------------------------------------------------- golden fixtures vs oracle
+def test_golden_notebook_blocks_match_oracle():
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "notebook_blocks.json")))
+    d = orc.notebook_inputs(np.float64)
+    R, C = g["mesh"]
+    full = {"os": orc.dense("os", d["X"], d["W"]), "ls": orc.dense("ls", d["dY"], d["W"]),
+            "rs": orc.dense("rs", d["X"], d["dY"])}
+    for flow, Y in full.items():
+        for key, st in g[flow].items():
+            i, j = map(int, key.split(","))
+            blk = orc.shard(Y, R, C, i, j)
+            assert blk.sum() == pytest.approx(st["sum"], rel=1e-13)
+            assert (blk * blk).sum() == pytest.approx(st["sumsq"], rel=1e-13)
+            assert [blk[0, 0], blk[0, -1], blk[-1, 0], blk[-1, -1]] == st["corners"]
