@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-device sliced GEMM on one MI355X.
+
+Workload (BASELINE config 2): GPT-3-like FFN up-projection, one device of a 4x4 mesh, output-stationary:
+X[4096,12288] bf16 ~N(0,1), W[12288,12288] bf16 ~N(0,0.02), S=4 block-cyclic slices along K (3072 each,
+materialised contiguous in HBM as an all-gather would deliver them), fp32 accumulate -> C[4096,12288] bf16.
+One "step" = one ms_gemm_os call over all four slices.  Inputs are resident in HBM before timing starts.
+
+Prints ONE JSON line: whole-job TFLOP/s (`value`), the kernel's roofline fraction measured with HIP events
+per launch (`roofline`), and the CPU restatement of the same device body timed on the host cores
+(`cpu_baseline`).  Extra keys report the S=1 baseline, the slicing overhead and the LS / RS configurations.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6     # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
+# HBM bytes per launch of the config-2 kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by
+# the same counters on a 1 GiB copy (see profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def sel_index(L, S, B, k):
+    g = np.arange(L)
+    return g[(g // B) % S == k]
+
+
+def make_config2(torch, S):
+    g = torch.Generator(device="cuda").manual_seed(0)
+    X = torch.randn((4096, 12288), generator=g, device="cuda").to(torch.bfloat16)
+    W = (torch.randn((12288, 12288), generator=g, device="cuda") * 0.02).to(torch.bfloat16)
+    idx = [torch.from_numpy(sel_index(12288, S, 8, k)).cuda() for k in range(S)]
+    A = [X[:, i].contiguous() for i in idx]
+    B = [W[i, :].contiguous() for i in idx]
+    return X, W, A, B
+
+
+def median(xs):
+    return float(np.median(np.asarray(xs, dtype=np.float64)))
+
+
+def cpu_baseline(A_host, B_host, flops_full):
+    """Time the oracle's CPU device body (per-slice fp32 BLAS loop) on a bounded sample."""
+    from oracle import meshslice_oracle as orc
+    try:
+        from threadpoolctl import threadpool_info, threadpool_limits
+    except Exception:  # pragma: no cover
+        threadpool_info = threadpool_limits = None
+    want = min(16, os.cpu_count() or 1)
+    ctx = threadpool_limits(limits=want) if threadpool_limits else None
+    try:
+        cores = want
+        if threadpool_info:
+            blas = [p for p in threadpool_info() if p.get("user_api") == "blas"]
+            if blas:
+                cores = int(blas[0].get("num_threads", want))
+        t0 = time.perf_counter()
+        orc.cpu_device_body_os(A_host[:1], B_host[:1])          # warm-up on one slice
+        t_one = time.perf_counter() - t0
+        S = len(A_host)
+        if t_one * S > 8.0:      # slow host: time a single slice, three times
+            reps, sample_slices = 3, 1
+        else:
+            reps, sample_slices = 3, S
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            orc.cpu_device_body_os(A_host[:sample_slices], B_host[:sample_slices])
+            ts.append(time.perf_counter() - t0)
+        sec = median(ts)
+        flops = flops_full * sample_slices / S
+        return {
+            "value": round(flops / sec / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{sample_slices} of {S} slices of the same workload ([4096,3072]x[3072,12288] each), fp32 BLAS on "
+                      f"bf16-rounded inputs, 1 warm-up + {reps} reps, median {sec:.3f} s; CPU restatement of the "
+                      f"reference device body (JAX is not installable offline)",
+            "seconds": round(sec, 4), "os_cpu_count": os.cpu_count(),
+        }
+    finally:
+        if ctx is not None:
+            ctx.__exit__(None, None, None)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one 1 GiB device copy (scales rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--only-main", action="store_true", help="skip the S=1 / LS / RS side measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures ONE mesh device's local GEMM on ONE GPU; --gpus > 1 is not part of this build "
+              "(the mesh is emulated on the host, no collectives are built).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import meshslice_amd as ms
+    from meshslice_amd import _lib
+    from oracle import meshslice_oracle as orc
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    lib = _lib.load()
+    torch.cuda.set_device(0)
+    S = 4
+    M, N, K = 4096, 12288, 12288
+    flops = 2.0 * M * N * K
+    X, W, A, B = make_config2(torch, S)
+    C = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    # ---- timed region: W warm-up steps, then exactly K steps between two synchronisations
+    for _ in range(args.warmup):
+        ms.gemm_os(A, B, out=C)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ms.gemm_os(A, B, out=C)
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = flops / (ms_per_step * 1e-3) / 1e12
+
+    # ---- kernel duration with HIP events around every launch, on the launch stream
+    per_launch = ms.time_call("os", (A, B), C, warmup=2, reps=max(args.steps, 10))
+    k_ms = float(np.mean(per_launch))
+    achieved = flops / (k_ms * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                "kernel_ms_mean": round(k_ms, 4), "kernel_ms_median": round(median(per_launch), 4),
+                "kernel_ms_min": round(float(np.min(per_launch)), 4),
+                "algorithmic_flops_per_launch": flops,
+                "algorithmic_hbm_bytes_per_launch": 2 * (M * K + K * N + M * N)}
+
+    extra = {}
+    # parity spot check of the benchmarked output against the float64 oracle on sampled rows
+    rows = np.random.default_rng(0).choice(M, 16, replace=False)
+    want = X[rows].float().cpu().numpy().astype(np.float64) @ W.float().cpu().numpy().astype(np.float64)
+    extra["parity_rel_frobenius_sampled_rows"] = float(f"{orc.rel_frobenius(C[rows].float().cpu().numpy(), want):.3e}")
+
+    if not args.only_main:
+        C1 = torch.empty_like(C)
+        t_s1 = median(ms.time_call("os", ([X], [W]), C1, warmup=3, reps=max(args.steps, 10)))
+        t_s4 = median(per_launch)
+        extra["os_s1_ms"] = round(t_s1, 4)
+        extra["os_s4_ms"] = round(t_s4, 4)
+        extra["slicing_overhead_s4_vs_s1"] = round(t_s4 / t_s1 - 1.0, 4)
+        del C1
+        # config 3: LS, S=8 -> 8 fp32 chunks [4096,1536]
+        idx8 = [torch.from_numpy(sel_index(12288, 8, 8, k)).cuda() for k in range(8)]
+        Ws = [W[i, :].contiguous() for i in idx8]
+        Y = [torch.empty((4096, 1536), dtype=torch.float32, device="cuda") for _ in range(8)]
+        t = median(ms.time_call("ls", (X, Ws), Y, warmup=3, reps=max(args.steps, 10)))
+        extra["ls_s8_ms"] = round(t, 4); extra["ls_s8_tflops"] = round(flops / t / 1e9, 1)
+        del Ws, Y
+        # config 4: RS, S=4 -> 4 fp32 chunks [768,12288]
+        g = torch.Generator(device="cuda").manual_seed(4)
+        X4 = torch.randn((4096, 3072), generator=g, device="cuda").to(torch.bfloat16)
+        dY = (torch.randn((4096, 12288), generator=g, device="cuda") * 1e-3).to(torch.bfloat16)
+        idx4 = [torch.from_numpy(sel_index(3072, 4, 8, k)).cuda() for k in range(4)]
+        Xs = [X4[:, i].contiguous() for i in idx4]
+        Y = [torch.empty((768, 12288), dtype=torch.float32, device="cuda") for _ in range(4)]
+        t = median(ms.time_call("rs", (Xs, dY), Y, warmup=3, reps=max(args.steps, 10)))
+        extra["rs_s4_ms"] = round(t, 4); extra["rs_s4_tflops"] = round(2.0 * 3072 * 12288 * 4096 / t / 1e9, 1)
+        del Xs, Y, X4, dY
+
+    out = {
+        "metric": "per-device sliced GEMM throughput (GPT-3 FFN up-proj, output-stationary, S=4)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "BASELINE config 2: one device of a 4x4 mesh, OS, X[4096,12288] x W[12288,12288] bf16, "
+                               "S=4 block-cyclic K slices of 3072, fp32 accumulate, C[4096,12288] bf16",
+                   "S": S, "m": M, "n": N, "k_slice": K // S, "blocksize": 8},
+        "pct_of_bf16_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        A_host = [a.float().cpu().numpy() for a in A]
+        B_host = [b.float().cpu().numpy() for b in B]
+        out["cpu_baseline"] = cpu_baseline(A_host, B_host, flops)
+    else:
+        out["cpu_baseline"] = None
+    out["extra"] = extra
+    out["device"] = {"cus": int(lib.ms_query(_lib.MS_QUERY_CU_COUNT)), "clock_khz": int(lib.ms_query(_lib.MS_QUERY_CLOCK_KHZ))}
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
