@@ -15,15 +15,16 @@
 
 // Every kernel variant is instantiated explicitly: with implicit instantiation alone the host
 // compiler leaves some of the launch stubs undefined.
-#define MS_INSTANTIATE(BM, BN, WGM, WGN)                                                                  \
-  template __global__ void msk::gemm_bf16_kernel<BM, BN, WGM, WGN, true, false, true>(const msk::GemmArgs);   \
-  template __global__ void msk::gemm_bf16_kernel<BM, BN, WGM, WGN, true, false, false>(const msk::GemmArgs);  \
-  template __global__ void msk::gemm_bf16_kernel<BM, BN, WGM, WGN, true, true, false>(const msk::GemmArgs);   \
-  template __global__ void msk::gemm_bf16_kernel<BM, BN, WGM, WGN, false, false, false>(const msk::GemmArgs);
-MS_INSTANTIATE(256, 256, 2, 2)
-MS_INSTANTIATE(256, 256, 2, 4)
-MS_INSTANTIATE(128, 128, 2, 2)
-#undef MS_INSTANTIATE
+#define MS_INSTANTIATE_RING(BM, BN, BK, NS, WGM, WGN)                                                                  \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, true>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, false>(const msk::GemmArgs);  \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, true, false>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, false, false, false>(const msk::GemmArgs);
+MS_INSTANTIATE_RING(256, 256, 64, 2, 2, 2)
+MS_INSTANTIATE_RING(256, 256, 32, 4, 2, 4)
+MS_INSTANTIATE_RING(128, 128, 64, 2, 2, 2)
+MS_INSTANTIATE_RING(256, 256, 32, 4, 2, 2)
+#undef MS_INSTANTIATE_RING
 
 namespace {
 
@@ -106,12 +107,13 @@ int validate(const Problem &p) {
   return MS_OK;
 }
 
-template <int BM, int BN, int WGM, int WGN, bool AK, bool BK_, bool OBF>
+template <int BM, int BN, int BK_, int NS, int WGM, int WGN, bool AK, bool BKM, bool OBF>
 void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
-  msk::gemm_bf16_kernel<BM, BN, WGM, WGN, AK, BK_, OBF><<<gd, bd, 0, stream>>>(g);
+  msk::gemm_bf16_ring_kernel<BM, BN, BK_, NS, WGM, WGN, AK, BKM, OBF><<<gd, bd, 0, stream>>>(g);
 }
 
-template <int BM, int BN, int WGM, int WGN>
+// tile BM x BN, WGM x WGN waves, NS ring stages of BK_ k-elements
+template <int BM, int BN, int WGM, int WGN, int BK_, int NS>
 int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
@@ -134,29 +136,33 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   dim3 gd(grid), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   if (p.flow == OS) {
-    if (obf) launch_one<BM, BN, WGM, WGN, true, false, true>(gd, bd, stream, g);
-    else launch_one<BM, BN, WGM, WGN, true, false, false>(gd, bd, stream, g);
+    if (obf) launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, true>(gd, bd, stream, g);
+    else launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, false>(gd, bd, stream, g);
   } else if (p.flow == LS) {
-    launch_one<BM, BN, WGM, WGN, true, true, false>(gd, bd, stream, g);
+    launch_one<BM, BN, BK_, NS, WGM, WGN, true, true, false>(gd, bd, stream, g);
   } else {
-    launch_one<BM, BN, WGM, WGN, false, false, false>(gd, bd, stream, g);
+    launch_one<BM, BN, BK_, NS, WGM, WGN, false, false, false>(gd, bd, stream, g);
   }
   MS_HIP(hipGetLastError());
   return MS_OK;
 }
 
+// Kernel variants.  1: 256x256 tile, 4 waves, 2 stages of 64; 2: 256x256, 8 waves, 4 stages of 32;
+// 3: 128x128, 4 waves, 2 stages of 64; 4: 256x256, 4 waves, 4 stages of 32.
 int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
   int v = g_variant;
   if (v == 0) {
-    // small outputs cannot fill 256 CUs with 256x256 tiles
     const long t256 = (long)((p.M + 255) / 256) * ((p.N + 255) / 256) * (p.flow == OS ? 1 : p.S);
-    v = t256 >= dev.cus ? 1 : 3;
+    if (t256 < dev.cus) v = 3;      // too few 256x256 tiles to fill the chip
+    else if (p.flow == LS) v = 1;   // both operands k-contiguous: 64-element stages fetch whole 128-byte lines
+    else v = 4;
   }
   switch (v) {
-    case 1: return launch_bf16_tile<256, 256, 2, 2>(p, dev, stream);
-    case 2: return launch_bf16_tile<256, 256, 2, 4>(p, dev, stream);
-    case 3: return launch_bf16_tile<128, 128, 2, 2>(p, dev, stream);
+    case 1: return launch_bf16_tile<256, 256, 2, 2, 64, 2>(p, dev, stream);
+    case 2: return launch_bf16_tile<256, 256, 2, 4, 32, 4>(p, dev, stream);
+    case 3: return launch_bf16_tile<128, 128, 2, 2, 64, 2>(p, dev, stream);
+    case 4: return launch_bf16_tile<256, 256, 2, 2, 32, 4>(p, dev, stream);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }
@@ -261,7 +267,7 @@ MS_API long ms_query(int what) {
 }
 
 MS_API int ms_set_variant(int variant) {
-  if (variant < 0 || variant > 3) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  if (variant < 0 || variant > 4) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
   g_variant = variant;
   return MS_OK;
 }
