@@ -163,3 +163,39 @@ def sweep_compute_term(meshes=((2, 8), (4, 4), (8, 8)), slice_counts=(1, 2, 4, 8
                         print(f"mesh {mesh[0]}x{mesh[1]} {lname:8s} {pname:10s} S={S:2d} {layout} "
                               f"[{M}x{N}x{K}] {seen[key]*1e3:.4f} ms/slice {tf:.0f} TFLOP/s", flush=True)
     return CostModel.fit_compute_term(samples), rows
+
+
+def _main(argv=None):
+    """``python -m meshslice_amd.Autotuner``: run the compute-term sweep on the GPU, print the table,
+    the fitted ``(t0, eta)`` per layout and the model's slice-count choice with the measured term."""
+    import argparse
+    import json
+    ap = argparse.ArgumentParser(description="refit the cost model's compute term from MI355X kernel times")
+    ap.add_argument("--passes", default="fwd", help="comma list of fwd,bwd_data,bwd_weight")
+    ap.add_argument("--slices", default="1,2,4,8,16")
+    ap.add_argument("--meshes", default="2x8,4x4,8x8")
+    ap.add_argument("--repeat", type=int, default=5)
+    ap.add_argument("--out", default=None, help="write the fitted term and the rows as JSON")
+    a = ap.parse_args(argv)
+    meshes = [tuple(int(v) for v in m.split("x")) for m in a.meshes.split(",")]
+    slices = [int(v) for v in a.slices.split(",")]
+    term, rows = sweep_compute_term(meshes, slices, tuple(a.passes.split(",")), repeat=a.repeat)
+    for lay in sorted(term.eta):
+        print(f"fit {lay}: t0 = {term.t0[lay]*1e6:.1f} us, eta = {term.eta[lay]:.3f} of {term.peak/1e12:.1f} TFLOP/s")
+    CostModel.use_compute_term(term)
+    try:
+        layers = [(B, I, O, df) for (_n, B, I, O, df) in gpt3_layers()]
+        for mesh in meshes:
+            total, best = emulateFFTime(layers, mesh, sweep=True, candidates=[s for s in slices if s > 1])
+            print(f"mesh {mesh[0]}x{mesh[1]}: model FF time {total*1e3:.3f} ms with slice counts {best} "
+                  f"(TPUv4 link constants of the reference, MI355X compute term)")
+    finally:
+        CostModel.use_compute_term(None)
+    if a.out:
+        with open(a.out, "w") as f:
+            json.dump({"term": term.to_dict(),
+                       "rows": [[f"{m[0]}x{m[1]}", ln, pn, S, M, N, K, lay, t] for (m, ln, pn, S, M, N, K, lay, t) in rows]}, f, indent=1)
+
+
+if __name__ == "__main__":
+    _main()
