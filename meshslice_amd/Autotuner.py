@@ -142,13 +142,14 @@ def per_slice_shapes(B, I, O, dataflow, meshshape, S, passes=("fwd", "bwd_data",
 
 
 def sweep_compute_term(meshes=((2, 8), (4, 4), (8, 8)), slice_counts=(1, 2, 4, 8, 16),
-                       passes=("fwd",), layers=None, repeat: int = 5, verbose: bool = True):
+                       passes=("fwd",), layers=None, repeat: int = 5, verbose: bool = True, fused: bool = False):
     """Measure every per-slice kernel of the sweep on the GPU and fit the compute term.
 
     Returns ``(ComputeTerm, rows)`` where each row is
-    ``(mesh, layer, pass, S, M, N, K, layout, seconds_per_slice)``."""
+    ``(mesh, layer, pass, S, M, N, K, layout, seconds_per_slice)``; with ``fused`` a tenth entry holds the
+    seconds of the one fused S-slice call a device really issues."""
     layers = layers or gpt3_layers()
-    rows, samples, seen = [], [], {}
+    rows, samples, seen, seen_fused = [], [], {}, {}
     for mesh in meshes:
         for (lname, B, I, O, dataflow) in layers:
             for S in slice_counts:
@@ -157,11 +158,20 @@ def sweep_compute_term(meshes=((2, 8), (4, 4), (8, 8)), slice_counts=(1, 2, 4, 8
                     if key not in seen:
                         seen[key] = CostModel.estimateMatmul(None, M, N, K, layout=layout, repeat=repeat)
                         samples.append((M, N, K, layout, seen[key]))
-                    rows.append((mesh, lname, pname, S, M, N, K, layout, seen[key]))
+                    row = (mesh, lname, pname, S, M, N, K, layout, seen[key])
+                    extra = ""
+                    if fused:
+                        fk = key + (S,)
+                        if fk not in seen_fused:
+                            seen_fused[fk] = CostModel.measureFused(M, N, K, S, layout=layout, repeat=repeat)
+                        row = row + (seen_fused[fk],)
+                        ftf = 2.0 * M * N * K * S / seen_fused[fk] / 1e12
+                        extra = f" | S x slice {S*seen[key]*1e3:.4f} ms, fused {seen_fused[fk]*1e3:.4f} ms {ftf:.0f} TFLOP/s"
+                    rows.append(row)
                     if verbose:
                         tf = 2.0 * M * N * K / seen[key] / 1e12
                         print(f"mesh {mesh[0]}x{mesh[1]} {lname:8s} {pname:10s} S={S:2d} {layout} "
-                              f"[{M}x{N}x{K}] {seen[key]*1e3:.4f} ms/slice {tf:.0f} TFLOP/s", flush=True)
+                              f"[{M}x{N}x{K}] {seen[key]*1e3:.4f} ms/slice {tf:.0f} TFLOP/s{extra}", flush=True)
     return CostModel.fit_compute_term(samples), rows
 
 
@@ -175,11 +185,12 @@ def _main(argv=None):
     ap.add_argument("--slices", default="1,2,4,8,16")
     ap.add_argument("--meshes", default="2x8,4x4,8x8")
     ap.add_argument("--repeat", type=int, default=5)
+    ap.add_argument("--fused", action="store_true", help="also time the fused S-slice call of every row")
     ap.add_argument("--out", default=None, help="write the fitted term and the rows as JSON")
     a = ap.parse_args(argv)
     meshes = [tuple(int(v) for v in m.split("x")) for m in a.meshes.split(",")]
     slices = [int(v) for v in a.slices.split(",")]
-    term, rows = sweep_compute_term(meshes, slices, tuple(a.passes.split(",")), repeat=a.repeat)
+    term, rows = sweep_compute_term(meshes, slices, tuple(a.passes.split(",")), repeat=a.repeat, fused=a.fused)
     for lay in sorted(term.eta):
         print(f"fit {lay}: t0 = {term.t0[lay]*1e6:.1f} us, eta = {term.eta[lay]:.3f} of {term.peak/1e12:.1f} TFLOP/s")
     CostModel.use_compute_term(term)
@@ -194,7 +205,7 @@ def _main(argv=None):
     if a.out:
         with open(a.out, "w") as f:
             json.dump({"term": term.to_dict(),
-                       "rows": [[f"{m[0]}x{m[1]}", ln, pn, S, M, N, K, lay, t] for (m, ln, pn, S, M, N, K, lay, t) in rows]}, f, indent=1)
+                       "rows": [[f"{r[0][0]}x{r[0][1]}"] + list(r[1:]) for r in rows]}, f, indent=1)
 
 
 if __name__ == "__main__":

@@ -139,6 +139,20 @@ def use_compute_term(term: Optional[ComputeTerm]) -> None:
     _installed = term
 
 
+def load_compute_term(path: Optional[str] = None) -> ComputeTerm:
+    """Install the compute term measured on MI355X that ships with the package (or the JSON at ``path``,
+    as written by ``python -m meshslice_amd.Autotuner --out``) and return it."""
+    import json
+    import os
+    if path is None:
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "data", "compute_term_mi355x.json")
+    with open(path) as f:
+        d = json.load(f)
+    term = ComputeTerm.from_dict(d["term"] if "term" in d else d)
+    use_compute_term(term)
+    return term
+
+
 def estimateMatmul(mesh, M, N, K, input_precision=None, layout: str = "nn", repeat: int = 5) -> float:
     """Seconds of one local ``[M,K] x [K,N]`` contraction (reference CostModel.py:74-98).
 
@@ -174,6 +188,32 @@ def estimateMatmul(mesh, M, N, K, input_precision=None, layout: str = "nn", repe
     sec = float(np.mean(ms)) * 1e-3
     _measured[key] = sec
     return sec
+
+
+def measureFused(M, N, K, S, layout: str = "nn", input_precision=None, repeat: int = 5) -> float:
+    """Seconds of ONE fused call that does the work of ``S`` per-slice contractions of shape
+    ``[M,K] x [K,N]`` (the per-slice shape ``estimateMatmul`` is asked about): 'nn' = ms_gemm_os over S
+    k-slices, 'nt' = ms_gemm_ls emitting S chunks, 'tn' = ms_gemm_rs emitting S chunks.  GPU only."""
+    import torch
+    from . import local_gemm
+    if layout not in ("nn", "nt", "tn"):
+        raise ValueError(f"unknown layout {layout!r}")
+    if not torch.cuda.is_available():
+        raise local_gemm._lib.MeshSliceError("measureFused needs the GPU")
+    dtype = input_precision or torch.bfloat16
+    M, N, K, S = int(M), int(N), int(K), int(S)
+    dev = "cuda"
+    ones = lambda *shape: torch.ones(shape, dtype=dtype, device=dev)
+    if layout == "nn":
+        A = [ones(M, K) for _ in range(S)]; B = [ones(K, N) for _ in range(S)]
+        ms = local_gemm.time_call("os", (A, B), torch.empty((M, N), dtype=dtype, device=dev), warmup=1, reps=repeat)
+    elif layout == "nt":
+        out = [torch.empty((M, N), dtype=torch.float32, device=dev) for _ in range(S)]
+        ms = local_gemm.time_call("ls", (ones(M, K), [ones(N, K) for _ in range(S)]), out, warmup=1, reps=repeat)
+    else:
+        out = [torch.empty((M, N), dtype=torch.float32, device=dev) for _ in range(S)]
+        ms = local_gemm.time_call("rs", ([ones(K, M) for _ in range(S)], ones(K, N)), out, warmup=1, reps=repeat)
+    return float(np.mean(ms)) * 1e-3
 
 
 # ------------------------------------------------------------------------------------------------

@@ -241,3 +241,17 @@ def test_golden_notebook_blocks_match_oracle():
             assert blk.sum() == pytest.approx(st["sum"], rel=1e-13)
             assert (blk * blk).sum() == pytest.approx(st["sumsq"], rel=1e-13)
             assert [blk[0, 0], blk[0, -1], blk[-1, 0], blk[-1, -1]] == st["corners"]
+
+
+def test_shipped_compute_term_loads_and_feeds_the_models():
+    term = CostModel.load_compute_term()
+    try:
+        assert set(term.eta) == {"nn", "nt", "tn"}
+        assert all(0.2 < e < 1.0 for e in term.eta.values())
+        # a measured point of the sweep: ff1 forward slice on the 4x4 mesh at S=4
+        t = CostModel.estimateMatmul(None, 4096, 12288, 3072, layout="nn")
+        assert 0.1e-3 < t < 0.5e-3
+        pro, steady = CostModel.MeshFlow_OS(_mesh((4, 4)), 16384, 49152, 12288, 4)
+        assert steady >= 4 * t
+    finally:
+        CostModel.use_compute_term(None)
