@@ -24,6 +24,8 @@ MS_INSTANTIATE_RING(256, 256, 64, 2, 2, 2)
 MS_INSTANTIATE_RING(256, 256, 32, 4, 2, 4)
 MS_INSTANTIATE_RING(128, 128, 64, 2, 2, 2)
 MS_INSTANTIATE_RING(256, 256, 32, 4, 2, 2)
+MS_INSTANTIATE_RING(256, 192, 32, 4, 2, 2)
+MS_INSTANTIATE_RING(192, 256, 32, 4, 2, 2)
 #undef MS_INSTANTIATE_RING
 
 namespace {
@@ -147,22 +149,37 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   return MS_OK;
 }
 
-// Kernel variants.  1: 256x256 tile, 4 waves, 2 stages of 64; 2: 256x256, 8 waves, 4 stages of 32;
-// 3: 128x128, 4 waves, 2 stages of 64; 4: 256x256, 4 waves, 4 stages of 32.
+// Kernel variants (tile, waves, ring stages x k-elements per stage):
+//   1: 256x256, 4 waves, 2 x 64     2: 256x256, 8 waves, 4 x 32     3: 128x128, 4 waves, 2 x 64
+//   4: 256x256, 4 waves, 4 x 32     5: 256x192, 4 waves, 4 x 32     6: 192x256, 4 waves, 4 x 32
+// The default picks the tile shape that wastes the least of the machine: a launch runs in
+// ceil(tiles / CUs) rounds of one tile per CU, so the estimate is rounds x tile area / relative tile
+// efficiency (measured on the GPT-3-sized product: 192-wide tiles reach 0.92 / 0.85 of the 256x256
+// rate, 128x128 tiles about 0.7).
 int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
   int v = g_variant;
   if (v == 0) {
-    const long t256 = (long)((p.M + 255) / 256) * ((p.N + 255) / 256) * (p.flow == OS ? 1 : p.S);
-    if (t256 < dev.cus) v = 3;      // too few 256x256 tiles to fill the chip
-    else if (p.flow == LS) v = 1;   // both operands k-contiguous: 64-element stages fetch whole 128-byte lines
-    else v = 4;
+    struct Cand { int v, bm, bn; double eff; };
+    const Cand cands[] = {{4, 256, 256, 1.0}, {5, 256, 192, 0.92}, {6, 192, 256, 0.85}, {3, 128, 128, 0.70}};
+    const long chunks = p.flow == OS ? 1 : p.S;
+    double best = 0;
+    for (const Cand &c : cands) {
+      const long tiles = (long)((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * chunks;
+      const long rounds = (tiles + dev.cus - 1) / dev.cus;
+      const double cost = (double)rounds * c.bm * c.bn / c.eff;
+      if (v == 0 || cost < best) { v = c.v; best = cost; }
+    }
+    // both operands k-contiguous: 64-element stages fetch whole 128-byte lines
+    if (v == 4 && p.flow == LS) v = 1;
   }
   switch (v) {
     case 1: return launch_bf16_tile<256, 256, 2, 2, 64, 2>(p, dev, stream);
     case 2: return launch_bf16_tile<256, 256, 2, 4, 32, 4>(p, dev, stream);
     case 3: return launch_bf16_tile<128, 128, 2, 2, 64, 2>(p, dev, stream);
     case 4: return launch_bf16_tile<256, 256, 2, 2, 32, 4>(p, dev, stream);
+    case 5: return launch_bf16_tile<256, 192, 2, 2, 32, 4>(p, dev, stream);
+    case 6: return launch_bf16_tile<192, 256, 2, 2, 32, 4>(p, dev, stream);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }
@@ -267,7 +284,7 @@ MS_API long ms_query(int what) {
 }
 
 MS_API int ms_set_variant(int variant) {
-  if (variant < 0 || variant > 4) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  if (variant < 0 || variant > 6) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
   g_variant = variant;
   return MS_OK;
 }
