@@ -278,3 +278,96 @@ def test_query_reports_the_device():
     assert lib.ms_query(_lib.MS_QUERY_CU_COUNT) == torch.cuda.get_device_properties(0).multi_processor_count
     assert lib.ms_query(_lib.MS_QUERY_LDS_BYTES) >= 160 * 1024
     assert lib.ms_query(1234) == -1
+
+
+# ------------------------------------------------------------------ streams, graphs, limits
+def test_non_default_stream_and_stream_ordering():
+    """Calls are asynchronous on the caller's stream: work queued on a side stream is ordered after the
+    producer on that stream and before the consumer."""
+    A, B = _rand_case("os", 512, 384, 256, 2, seed=21, dtype=torch.bfloat16)
+    want = orc.oracle_os_block(A, B)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        a = [dev(x, torch.bfloat16) for x in A]; b = [dev(x, torch.bfloat16) for x in B]
+        out = ms.gemm_os(a, b, out_dtype=torch.float32)
+        doubled = out * 2
+    torch.cuda.current_stream().wait_stream(side)
+    assert orc.rel_frobenius(host(doubled), 2 * want) <= TOL_BF16
+
+
+def test_hip_graph_capture_and_replay():
+    """The entry points launch kernels only (no allocation, no memset), so they can be captured; every
+    replay is checked against the eager result, with eager work in between."""
+    A, W = _rand_case("ls", 384, 256, 320, 3, seed=22, dtype=torch.bfloat16)
+    a = dev(A, torch.bfloat16); ws = [dev(w, torch.bfloat16) for w in W]
+    eager = [t.clone() for t in ms.gemm_ls(a, ws)]
+    outs = [torch.zeros_like(t) for t in eager]
+    ms.gemm_ls(a, ws, out=outs)                      # warm-up outside capture
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        ms.gemm_ls(a, ws, out=outs)
+    for rep in range(3):
+        for t in outs:
+            t.zero_()
+        scratch = ms.gemm_os([a], [ws[0].t().contiguous()])   # eager work between replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, eager):
+            assert torch.equal(got, want), f"replay {rep} differs from the eager result"
+        del scratch
+
+
+def test_maximum_slice_count_and_one_beyond():
+    S = 64
+    A, B = _rand_case("os", 72, 136, 16, S, seed=23, dtype=torch.bfloat16)
+    _run_and_compare("os", (A, B), torch.bfloat16, TOL_BF16)
+    X, W = _rand_case("rs", 40, 264, 24, S, seed=24, dtype=torch.bfloat16)
+    _run_and_compare("rs", (X, W), torch.bfloat16, TOL_BF16)
+    a = [dev(x, torch.bfloat16) for x in A] + [dev(A[0], torch.bfloat16)]
+    b = [dev(x, torch.bfloat16) for x in B] + [dev(B[0], torch.bfloat16)]
+    with pytest.raises(ValueError, match="S = 65"):
+        ms.gemm_os(a, b)
+
+
+def test_concurrent_host_threads_on_separate_streams():
+    import threading
+    cases = [_rand_case("os", 256 + 8 * t, 264, 128, 2, seed=30 + t, dtype=torch.bfloat16) for t in range(4)]
+    results, errors = [None] * 4, []
+
+    def work(t):
+        try:
+            torch.cuda.set_device(0)
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                A, B = cases[t]
+                for _ in range(5):
+                    out = ms.gemm_os([dev(x, torch.bfloat16) for x in A], [dev(x, torch.bfloat16) for x in B],
+                                     out_dtype=torch.float32)
+                st.synchronize()
+                results[t] = host(out)
+        except Exception as e:  # pragma: no cover
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors
+    for t in range(4):
+        assert orc.rel_frobenius(results[t], orc.oracle_os_block(*cases[t])) <= TOL_BF16
+
+
+def test_nan_and_inf_propagate():
+    A, B = _rand_case("os", 64, 64, 64, 1, seed=40, dtype=torch.bfloat16)
+    A[0][3, 5] = np.nan
+    B[0][7, 9] = np.inf
+    got = host(ms.gemm_os([dev(A[0], torch.bfloat16)], [dev(B[0], torch.bfloat16)], out_dtype=torch.float32))
+    assert np.isnan(got[3]).all()                    # a NaN in row 3 of A poisons row 3 of C
+    col = np.delete(got[:, 9], 3)
+    assert np.isinf(col).all() or np.isnan(col).any() is False and np.isinf(col).all()
+    clean = np.delete(np.delete(got, 3, axis=0), 9, axis=1)
+    assert np.isfinite(clean).all()
