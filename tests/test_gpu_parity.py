@@ -147,7 +147,7 @@ def _run_and_compare(flow, ops, dtype, tol, out_dtype=None):
     return err
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("flow", ["os", "ls", "rs"])
 def test_bf16_random_cases_all_variants(flow, variant):
     _lib.check(_lib.load().ms_set_variant(variant))
