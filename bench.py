@@ -180,6 +180,20 @@ def main():
         t = median(ms.time_call("rs", (Xs, dY), Y, warmup=3, reps=max(args.steps, 10)))
         extra["rs_s4_ms"] = round(t, 4); extra["rs_s4_tflops"] = round(2.0 * 3072 * 12288 * 4096 / t / 1e9, 1)
         del Xs, Y, X4, dY
+        # fused epilogue: GELU folded into the config-2 product vs the product followed by a separate GELU kernel
+        def _events(f, n):
+            for _ in range(3):
+                f()
+            torch.cuda.synchronize()
+            ts = []
+            for _ in range(n):
+                e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+                e0.record(); f(); e1.record(); torch.cuda.synchronize()
+                ts.append(e0.elapsed_time(e1))
+            return median(ts)
+        extra["os_s4_fused_gelu_ms"] = round(_events(lambda: ms.gemm_os(A, B, out=C, activation="gelu"), 10), 4)
+        extra["os_s4_then_separate_gelu_ms"] = round(_events(
+            lambda: torch.nn.functional.gelu(ms.gemm_os(A, B, out=C), approximate="tanh"), 10), 4)
 
     out = {
         "metric": "per-device sliced GEMM throughput (GPT-3 FFN up-proj, output-stationary, S=4)",

@@ -62,6 +62,26 @@ int ms_gemm_os(const void *const *A_slices, const void *const *B_slices, int S,
                int m, int n, int k_slice, int lda, int ldb,
                void *C, int ldc, int in_dtype, int out_dtype, void *stream);
 
+/* Output-stationary with a fused epilogue (bf16 operands only):
+ *     Y = act(sum_s A_s @ B_s) + residual          (fp32, then one rounding to out_dtype into C)
+ *     row_sum[i]   += sum_j Y[i,j]                 (optional, fp32 atomics)
+ *     row_sumsq[i] += sum_j Y[i,j]^2               (optional, fp32 atomics)
+ * Folds into the local product the element-wise work the reference's transformer block does right
+ * after an output-stationary layer: the GELU after ff1 (reference ShardedLayers.py:181-182), the
+ * residual add before a layer norm (:178,:184) and that norm's local row moments, which the mesh
+ * then sums over its columns (mn_l / sqmn_l, :125-126: divide by n for the means).
+ * activation: MS_ACT_NONE or MS_ACT_GELU (tanh form, the default of jax.nn.gelu).  residual: [m,n] in
+ * out_dtype with leading dimension ldr, or NULL.  row_sum / row_sumsq: [m] fp32 vectors the caller has
+ * zeroed, or NULL; the order of the atomic additions is not fixed, so their last bits can differ from
+ * run to run. */
+#define MS_ACT_NONE 0
+#define MS_ACT_GELU 1
+int ms_gemm_os_fused(const void *const *A_slices, const void *const *B_slices, int S,
+                     int m, int n, int k_slice, int lda, int ldb,
+                     void *C, int ldc, int in_dtype, int out_dtype,
+                     int activation, const void *residual, int ldr,
+                     float *row_sum, float *row_sumsq, void *stream);
+
 /* LHS-stationary: for s < S, Y_s[m,n_slice] = A[m,k] @ W_s[n_slice,k]^T  (fp32 out).
  * Replaces the contractions of MeshFlow_LS (TensorParallel.py:181,187); S == 1 is Collective_LS
  * (TensorParallel.py:26).  A is the device's own shard; W_s the s-th all-gathered row slice of the

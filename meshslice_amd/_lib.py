@@ -21,13 +21,15 @@ MS_QUERY_CLOCK_KHZ = 1
 MS_QUERY_IS_GFX950 = 2
 MS_QUERY_LDS_BYTES = 3
 MS_QUERY_MAX_SLICES = 4
+MS_ACT_NONE = 0
+MS_ACT_GELU = 1
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmeshslice_hip.so")
 
 EXPORTS = (
     "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
-    "ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs",
+    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_ls", "ms_gemm_rs",
     "ms_time_os", "ms_time_ls", "ms_time_rs",
 )
 
@@ -54,6 +56,8 @@ def _declare(lib):
     os_args = [vpp, vpp, c_int, c_int, c_int, c_int, c_int, c_int, c_vp, c_int, c_int, c_int, c_vp]
     ls_args = [c_vp, c_int, vpp, c_int, c_int, c_int, c_int, c_int, vpp, c_int, c_int, c_vp]
     rs_args = [vpp, c_int, c_vp, c_int, c_int, c_int, c_int, c_int, vpp, c_int, c_int, c_vp]
+    lib.ms_gemm_os_fused.argtypes = os_args[:-1] + [c_int, c_vp, c_int, c_vp, c_vp, c_vp]
+    lib.ms_gemm_os_fused.restype = c_int
     lib.ms_gemm_os.argtypes = os_args
     lib.ms_gemm_ls.argtypes = ls_args
     lib.ms_gemm_rs.argtypes = rs_args

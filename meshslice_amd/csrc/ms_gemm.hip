@@ -15,11 +15,13 @@
 
 // Every kernel variant is instantiated explicitly: with implicit instantiation alone the host
 // compiler leaves some of the launch stubs undefined.
-#define MS_INSTANTIATE_RING(BM, BN, BK, NS, WGM, WGN)                                                                  \
-  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, true>(const msk::GemmArgs);   \
-  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, false>(const msk::GemmArgs);  \
-  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, true, false>(const msk::GemmArgs);   \
-  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, false, false, false>(const msk::GemmArgs);
+#define MS_INSTANTIATE_RING(BM, BN, BK, NS, WGM, WGN)                                                                         \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, true, false>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, false, false>(const msk::GemmArgs);  \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, true, true>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, false, true>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, true, false, false>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, false, false, false, false>(const msk::GemmArgs);
 MS_INSTANTIATE_RING(256, 256, 64, 2, 2, 2)
 MS_INSTANTIATE_RING(256, 256, 32, 4, 2, 4)
 MS_INSTANTIATE_RING(128, 128, 64, 2, 2, 2)
@@ -83,6 +85,12 @@ struct Problem {
   int M, N, K;           // per-chunk rows/cols, per-slice contraction
   int lda, ldb, ldc;
   int in_dtype, out_dtype;
+  // fused OS epilogue (all zero / null = plain product)
+  int act = 0;
+  const void *res = nullptr;
+  int ldr = 0;
+  float *row_sum = nullptr;
+  float *row_sumsq = nullptr;
 };
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -104,15 +112,23 @@ int validate(const Problem &p) {
   if (p.lda % q || p.ldb % q) return fail(MS_ERR_ARG, "%s: operand leading dimensions must be multiples of %d", fn, q);
   const int qo = p.out_dtype == MS_DTYPE_BF16 ? 8 : 4;
   if (p.N % qo || p.ldc % qo) return fail(MS_ERR_ARG, "%s: output columns / leading dimension must be multiples of %d", fn, qo);
+  if (p.act != MS_ACT_NONE && p.act != MS_ACT_GELU) return fail(MS_ERR_ARG, "%s: unknown activation %d", fn, p.act);
+  if (p.res) {
+    if (!aligned16(p.res)) return fail(MS_ERR_ARG, "%s: residual pointer not 16-byte aligned", fn);
+    if (p.ldr < p.N || p.ldr % qo) return fail(MS_ERR_ARG, "%s: residual leading dimension %d must be >= n and a multiple of %d", fn, p.ldr, qo);
+  }
+  if ((reinterpret_cast<uintptr_t>(p.row_sum) | reinterpret_cast<uintptr_t>(p.row_sumsq)) & 3) return fail(MS_ERR_ARG, "%s: row-moment pointers must be 4-byte aligned", fn);
+  if ((p.act || p.res || p.row_sum || p.row_sumsq) && (p.flow != OS || p.in_dtype != MS_DTYPE_BF16))
+    return fail(MS_ERR_UNSUPPORTED, "%s: the fused epilogue exists for the output-stationary bf16 kernel only", fn);
   for (int i = 0; i < p.na; i++) if (!p.a[i] || !aligned16(p.a[i])) return fail(MS_ERR_ARG, "%s: operand pointer %d null or not 16-byte aligned", fn, i);
   for (int i = 0; i < p.nb; i++) if (!p.b[i] || !aligned16(p.b[i])) return fail(MS_ERR_ARG, "%s: operand pointer %d null or not 16-byte aligned", fn, i);
   for (int i = 0; i < p.nc; i++) if (!p.c[i] || !aligned16(p.c[i])) return fail(MS_ERR_ARG, "%s: output pointer %d null or not 16-byte aligned", fn, i);
   return MS_OK;
 }
 
-template <int BM, int BN, int BK_, int NS, int WGM, int WGN, bool AK, bool BKM, bool OBF>
+template <int BM, int BN, int BK_, int NS, int WGM, int WGN, bool AK, bool BKM, bool OBF, bool EPI>
 void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
-  msk::gemm_bf16_ring_kernel<BM, BN, BK_, NS, WGM, WGN, AK, BKM, OBF><<<gd, bd, 0, stream>>>(g);
+  msk::gemm_bf16_ring_kernel<BM, BN, BK_, NS, WGM, WGN, AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
 }
 
 // tile BM x BN, WGM x WGN waves, NS ring stages of BK_ k-elements
@@ -138,13 +154,20 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   int grid = dev.cus < g.total_tiles ? dev.cus : g.total_tiles;
   dim3 gd(grid), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
+  g.act = p.act; g.res = p.res; g.ldr = p.ldr; g.row_sum = p.row_sum; g.row_sumsq = p.row_sumsq;
+  const bool epi = p.act != 0 || p.res || p.row_sum || p.row_sumsq;
   if (p.flow == OS) {
-    if (obf) launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, true>(gd, bd, stream, g);
-    else launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, false>(gd, bd, stream, g);
+    if (epi) {
+      if (obf) launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, true, true>(gd, bd, stream, g);
+      else launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, false, true>(gd, bd, stream, g);
+    } else {
+      if (obf) launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, true, false>(gd, bd, stream, g);
+      else launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, false, false>(gd, bd, stream, g);
+    }
   } else if (p.flow == LS) {
-    launch_one<BM, BN, BK_, NS, WGM, WGN, true, true, false>(gd, bd, stream, g);
+    launch_one<BM, BN, BK_, NS, WGM, WGN, true, true, false, false>(gd, bd, stream, g);
   } else {
-    launch_one<BM, BN, BK_, NS, WGM, WGN, false, false, false>(gd, bd, stream, g);
+    launch_one<BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
   }
   MS_HIP(hipGetLastError());
   return MS_OK;
@@ -249,23 +272,25 @@ int timed(const Problem &p, void *stream, int warmup, int reps, float *ms_out) {
   return rc;
 }
 
+Problem make_problem(Flow flow, const void *const *a, const void *const *b, void *const *c, int na, int nb, int nc, int S,
+                     int m, int n, int k, int lda, int ldb, int ldc, int in_dtype, int out_dtype) {
+  Problem p;
+  p.flow = flow; p.a = a; p.b = b; p.c = c; p.na = na; p.nb = nb; p.nc = nc; p.S = S;
+  p.M = m; p.N = n; p.K = k; p.lda = lda; p.ldb = ldb; p.ldc = ldc; p.in_dtype = in_dtype; p.out_dtype = out_dtype;
+  if (S < 1 || S > MS_MAX_SLICES) p.na = p.nb = p.nc = 0;   // the pointer tables are not read for a bad S
+  return p;
+}
 Problem make_os(const void *const *A, const void *const *B, int S, int m, int n, int k, int lda, int ldb,
                 void *const *C, int ldc, int in_dtype, int out_dtype) {
-  Problem p{OS, A, B, C, S, S, 1, S, m, n, k, lda, ldb, ldc, in_dtype, out_dtype};
-  if (S < 1 || S > MS_MAX_SLICES) p.na = p.nb = 0;
-  return p;
+  return make_problem(OS, A, B, C, S, S, 1, S, m, n, k, lda, ldb, ldc, in_dtype, out_dtype);
 }
 Problem make_ls(const void *const *A, int lda, const void *const *W, int ldw, int S, int m, int n, int k,
                 float *const *Y, int ldy, int in_dtype) {
-  Problem p{LS, A, W, (void *const *)Y, 1, S, S, S, m, n, k, lda, ldw, ldy, in_dtype, MS_DTYPE_F32};
-  if (S < 1 || S > MS_MAX_SLICES) p.nb = p.nc = 0;
-  return p;
+  return make_problem(LS, A, W, (void *const *)Y, 1, S, S, S, m, n, k, lda, ldw, ldy, in_dtype, MS_DTYPE_F32);
 }
 Problem make_rs(const void *const *X, int ldx, const void *const *W, int ldw, int S, int m, int n, int k,
                 float *const *Y, int ldy, int in_dtype) {
-  Problem p{RS, X, W, (void *const *)Y, S, 1, S, S, m, n, k, ldx, ldw, ldy, in_dtype, MS_DTYPE_F32};
-  if (S < 1 || S > MS_MAX_SLICES) p.na = p.nc = 0;
-  return p;
+  return make_problem(RS, X, W, (void *const *)Y, S, 1, S, S, m, n, k, ldx, ldw, ldy, in_dtype, MS_DTYPE_F32);
 }
 
 }  // namespace
@@ -297,6 +322,15 @@ MS_API int ms_gemm_os(const void *const *A_slices, const void *const *B_slices, 
                       int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype, void *stream) {
   void *c1[1] = {C};
   return run(make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype), stream);
+}
+
+MS_API int ms_gemm_os_fused(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
+                            int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype, int activation,
+                            const void *residual, int ldr, float *row_sum, float *row_sumsq, void *stream) {
+  void *c1[1] = {C};
+  Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
+  p.act = activation; p.res = residual; p.ldr = ldr; p.row_sum = row_sum; p.row_sumsq = row_sumsq;
+  return run(p, stream);
 }
 
 MS_API int ms_gemm_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,

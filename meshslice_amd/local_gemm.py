@@ -46,8 +46,14 @@ def _same(ts: Sequence[torch.Tensor], name: str):
 
 
 def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
-            out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """``C = sum_s A_s @ B_s`` with fp32 accumulation over all slices, rounded once."""
+            out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
+            activation: Optional[str] = None, residual: Optional[torch.Tensor] = None,
+            row_moments=None) -> torch.Tensor:
+    """``C = sum_s A_s @ B_s`` with fp32 accumulation over all slices, rounded once.
+
+    Optional fused epilogue (bf16 operands): ``C = act(sum) + residual`` with ``activation='gelu'`` (tanh
+    form) and ``residual`` of C's shape and dtype; ``row_moments=(row_sum, row_sumsq)`` are fp32 vectors of
+    length m (either may be None) to which the row sums / sums of squares of the fp32 result are ADDED."""
     a0 = _same(A_slices, "A_slices"); b0 = _same(B_slices, "B_slices")
     if len(A_slices) != len(B_slices):
         raise ValueError("A_slices and B_slices differ in length")
@@ -61,9 +67,32 @@ def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
         raise ValueError("out has the wrong shape")
     pa, _ka = _lib.ptr_array([t.data_ptr() for t in A_slices])
     pb, _kb = _lib.ptr_array([t.data_ptr() for t in B_slices])
+    fused = activation is not None or residual is not None or row_moments is not None
+    if not fused:
+        with torch.cuda.device(a0.device):
+            rc = _lib.load().ms_gemm_os(pa, pb, len(A_slices), m, n, k, a0.stride(0), b0.stride(0),
+                                        ctypes.c_void_p(out.data_ptr()), out.stride(0), _dt(a0), _dt(out), _stream())
+        _lib.check(rc)
+        return out
+    if activation not in (None, "gelu"):
+        raise ValueError(f"unknown activation {activation!r} (None or 'gelu')")
+    res_ptr, ldr = None, 0
+    if residual is not None:
+        _check2d(residual, "residual")
+        if tuple(residual.shape) != (m, n) or residual.dtype != out.dtype:
+            raise ValueError("residual must have the shape and dtype of the output")
+        res_ptr, ldr = ctypes.c_void_p(residual.data_ptr()), residual.stride(0)
+    moments = [None, None]
+    for idx, t in enumerate(row_moments or (None, None)):
+        if t is not None:
+            if not (t.is_cuda and t.dtype == torch.float32 and t.dim() == 1 and t.numel() == m and t.is_contiguous()):
+                raise ValueError("row moments must be contiguous fp32 GPU vectors of length m")
+            moments[idx] = ctypes.c_void_p(t.data_ptr())
     with torch.cuda.device(a0.device):
-        rc = _lib.load().ms_gemm_os(pa, pb, len(A_slices), m, n, k, a0.stride(0), b0.stride(0),
-                                    ctypes.c_void_p(out.data_ptr()), out.stride(0), _dt(a0), _dt(out), _stream())
+        rc = _lib.load().ms_gemm_os_fused(pa, pb, len(A_slices), m, n, k, a0.stride(0), b0.stride(0),
+                                          ctypes.c_void_p(out.data_ptr()), out.stride(0), _dt(a0), _dt(out),
+                                          _lib.MS_ACT_GELU if activation == "gelu" else _lib.MS_ACT_NONE,
+                                          res_ptr, ldr, moments[0], moments[1], _stream())
     _lib.check(rc)
     return out
 

@@ -194,6 +194,28 @@ def oracle_rs_chunks(X_slices, W):
     return [np.asarray(x, np.float64).T @ w for x in X_slices]
 
 
+def gelu_tanh(x: np.ndarray) -> np.ndarray:
+    """GELU in the tanh form ``0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))`` in float64: what
+    ``jax.nn.gelu`` computes by default, applied by the reference after ff1 (ShardedLayers.py:182)."""
+    x = np.asarray(x, np.float64)
+    return 0.5 * x * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (x + 0.044715 * x ** 3)))
+
+
+def oracle_os_fused(A_slices, B_slices, activation=None, residual=None):
+    """Float64 oracle of the output-stationary block with the element-wise work that follows it in the
+    reference's transformer block folded in: ``Y = act(sum_k A_k @ B_k) + residual`` (ShardedLayers.py:181-184)
+    and the local row moments of ``Y`` that the layer norm sums over the mesh columns (:125-126, as sums).
+    Returns ``(Y, row_sum, row_sumsq)``."""
+    y = oracle_os_block(A_slices, B_slices)
+    if activation == "gelu":
+        y = gelu_tanh(y)
+    elif activation is not None:
+        raise ValueError(f"unknown activation {activation!r}")
+    if residual is not None:
+        y = y + np.asarray(residual, np.float64)
+    return y, y.sum(axis=1), (y * y).sum(axis=1)
+
+
 def assemble_ls(chunks_by_col, R, C, j, S, B):
     """Mesh completion of LS for device column j: ``chunks_by_col[j'][k]`` are the partial
     chunks ``[m, O/S]`` of the C devices of one mesh row.  psum_scatter over ``col`` along

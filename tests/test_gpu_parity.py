@@ -371,3 +371,48 @@ def test_nan_and_inf_propagate():
     assert np.isinf(col).all() or np.isnan(col).any() is False and np.isinf(col).all()
     clean = np.delete(np.delete(got, 3, axis=0), 9, axis=1)
     assert np.isfinite(clean).all()
+
+
+# ------------------------------------------------------------------ fused output-stationary epilogue
+@pytest.mark.parametrize("variant", [0, 3, 4, 5, 7])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_fused_epilogue_gelu_residual_moments(variant, out_dtype):
+    """ms_gemm_os_fused: Y = gelu(sum_k A_k B_k) + residual, plus the row sums / sums of squares of Y
+    (the local layer-norm moments of reference ShardedLayers.py:125-126) against the float64 oracle."""
+    _lib.check(_lib.load().ms_set_variant(variant))
+    m, n, k, S = 520, 776, 136, 3
+    A, B = _rand_case("os", m, n, k, S, seed=50 + variant, dtype=torch.bfloat16)
+    rng = np.random.default_rng(99)
+    R = rng.standard_normal((m, n)).astype(np.float32)
+    R = orc.bf16_round(R) if out_dtype == torch.bfloat16 else R
+    a = [dev(x, torch.bfloat16) for x in A]; b = [dev(x, torch.bfloat16) for x in B]
+    s1 = torch.zeros(m, device="cuda"); s2 = torch.zeros(m, device="cuda")
+    got = ms.gemm_os(a, b, out_dtype=out_dtype, activation="gelu", residual=dev(R, out_dtype), row_moments=(s1, s2))
+    want, w1, w2 = orc.oracle_os_fused(A, B, "gelu", R)
+    tol = TOL_BF16 if out_dtype == torch.bfloat16 else 1e-5
+    assert orc.rel_frobenius(host(got), want) <= tol
+    assert orc.rel_frobenius(host(s1), w1) <= 1e-4          # moments come from the fp32 values before rounding
+    assert orc.rel_frobenius(host(s2), w2) <= 1e-4
+    # each part alone
+    plain = ms.gemm_os(a, b, out_dtype=torch.float32)
+    only_act = ms.gemm_os(a, b, out_dtype=torch.float32, activation="gelu")
+    assert orc.rel_frobenius(host(only_act), orc.gelu_tanh(host(plain))) <= 1e-6
+    only_res = ms.gemm_os(a, b, out_dtype=torch.float32, residual=dev(R.astype(np.float32), torch.float32))
+    assert torch.equal(only_res, plain + dev(R.astype(np.float32), torch.float32))
+    s1b = torch.zeros(m, device="cuda")
+    again = ms.gemm_os(a, b, out_dtype=torch.float32, row_moments=(s1b, None))
+    assert torch.equal(again, plain)
+    assert orc.rel_frobenius(host(s1b), host(plain).sum(1)) <= 1e-4
+
+
+def test_fused_epilogue_rejections():
+    a = torch.zeros((64, 64), dtype=torch.float32, device="cuda")
+    with pytest.raises(_lib.MeshSliceError):                 # fp32 operands: no fused kernel
+        ms.gemm_os([a], [a], activation="gelu")
+    h = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        ms.gemm_os([h], [h], activation="relu")
+    with pytest.raises(ValueError):
+        ms.gemm_os([h], [h], residual=torch.zeros((64, 32), dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        ms.gemm_os([h], [h], row_moments=(torch.zeros(63, device="cuda"), None))

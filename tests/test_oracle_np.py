@@ -254,3 +254,30 @@ def test_vjp_permutation_matches_autograd(dataflow):
         dx, dw = orc.dense("ls", wn, dyn), orc.dense("os", xn, dyn)
     assert np.allclose(dx, x.grad.numpy(), rtol=1e-12, atol=1e-12)
     assert np.allclose(dw, w.grad.numpy(), rtol=1e-12, atol=1e-12)
+
+
+# ---------------------------------------------------------------- fused epilogue oracle
+def test_gelu_tanh_matches_torch_and_identities():
+    x = np.concatenate([np.linspace(-12, 12, 4001), [0.0, 1e-8, -1e-8, 30.0, -30.0]])
+    want = torch.nn.functional.gelu(torch.from_numpy(x), approximate="tanh").numpy()
+    got = orc.gelu_tanh(x)
+    assert np.allclose(got, want, rtol=1e-13, atol=1e-15)
+    assert orc.gelu_tanh(0.0) == 0.0
+    assert np.allclose(orc.gelu_tanh(x) - orc.gelu_tanh(-x), x, rtol=1e-13, atol=1e-15)   # x*Phi(x) - (-x)*Phi(-x) = x
+    assert orc.gelu_tanh(30.0) == 30.0 and orc.gelu_tanh(-30.0) == 0.0
+    assert orc.gelu_tanh(1.0) == pytest.approx(0.8411919906082768, rel=1e-14)             # 0.5*(1+tanh(sqrt(2/pi)*1.044715))
+
+
+def test_oracle_os_fused_composes_the_parts():
+    rng = np.random.default_rng(8)
+    A = [rng.integers(-3, 4, (6, 8)).astype(np.float64) for _ in range(2)]
+    B = [rng.integers(-3, 4, (8, 5)).astype(np.float64) * 0.25 for _ in range(2)]
+    R = rng.integers(-3, 4, (6, 5)).astype(np.float64)
+    y, s1, s2 = orc.oracle_os_fused(A, B, "gelu", R)
+    base = A[0] @ B[0] + A[1] @ B[1]
+    assert np.array_equal(y, orc.gelu_tanh(base) + R)
+    assert np.allclose(s1, y.sum(1)) and np.allclose(s2, (y ** 2).sum(1))
+    y0, _, _ = orc.oracle_os_fused(A, B)
+    assert np.array_equal(y0, base)
+    with pytest.raises(ValueError):
+        orc.oracle_os_fused(A, B, "relu")
