@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the per-device sliced GEMM on one MI355X.
 
-Workload (BASELINE config 2): GPT-3-like FFN up-projection, one device of a 4x4 mesh, output-stationary:
+Workload (the headline configuration): GPT-3-like FFN up-projection, one device of a 4x4 mesh, output-stationary:
 X[4096,12288] bf16 ~N(0,1), W[12288,12288] bf16 ~N(0,0.02), S=4 block-cyclic slices along K (3072 each,
 materialised contiguous in HBM as an all-gather would deliver them), fp32 accumulate -> C[4096,12288] bf16.
 One "step" = one ms_gemm_os call over all four slices.  Inputs are resident in HBM before timing starts.
@@ -200,7 +200,7 @@ def main():
         "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "BASELINE config 2: one device of a 4x4 mesh, OS, X[4096,12288] x W[12288,12288] bf16, "
+        "config": {"workload": "GPT-3-like FFN up-projection: one device of a 4x4 mesh, OS, X[4096,12288] x W[12288,12288] bf16, "
                                "S=4 block-cyclic K slices of 3072, fp32 accumulate, C[4096,12288] bf16",
                    "S": S, "m": M, "n": N, "k_slice": K // S, "blocksize": 8},
         "pct_of_bf16_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),

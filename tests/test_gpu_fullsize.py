@@ -1,4 +1,4 @@
-"""BASELINE configs 2-4 at their full sizes, checked through size-independent properties: sampled
+"""The three GPT-3-sized configurations (output-, LHS- and RHS-stationary) at their full sizes, checked through size-independent properties: sampled
 rows / columns against the float64 oracle, slice-count invariance (S slices give the unsliced product),
 linearity in one operand, and chunk independence."""
 import numpy as np

@@ -41,7 +41,7 @@ def _default_variant():
     torch.cuda.synchronize()
 
 
-# ------------------------------------------------------------------ BASELINE config 1 (fp32 plumbing check)
+# ------------------------------------------------------------------ the fp32 plumbing configuration (2x2 mesh, 1024^2, S=4)
 def test_config1_fp32_os_device00_matches_oracle():
     rng = np.random.default_rng(0)
     A = rng.standard_normal((1024, 1024)).astype(np.float32)
