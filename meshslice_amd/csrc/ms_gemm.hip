@@ -29,6 +29,8 @@ MS_INSTANTIATE_RING(256, 256, 32, 4, 2, 2)
 MS_INSTANTIATE_RING(256, 192, 32, 4, 2, 2)
 MS_INSTANTIATE_RING(192, 256, 32, 4, 2, 2)
 MS_INSTANTIATE_RING(256, 256, 64, 2, 2, 4)
+MS_INSTANTIATE_RING(256, 192, 64, 2, 2, 2)
+MS_INSTANTIATE_RING(192, 256, 64, 2, 2, 2)
 #undef MS_INSTANTIATE_RING
 
 namespace {
@@ -176,17 +178,18 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
 // Kernel variants (tile, waves, ring stages x k-elements per stage):
 //   1: 256x256, 4 waves, 2 x 64     2: 256x256, 8 waves, 4 x 32     3: 128x128, 4 waves, 2 x 64
 //   4: 256x256, 4 waves, 4 x 32     5: 256x192, 4 waves, 4 x 32     6: 192x256, 4 waves, 4 x 32
-//   7: 256x256, 8 waves, 2 x 64
+//   7: 256x256, 8 waves, 2 x 64     8: 256x192, 4 waves, 2 x 64     9: 192x256, 4 waves, 2 x 64
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
 // ceil(tiles / CUs) rounds of one tile per CU, so the estimate is rounds x tile area / relative tile
-// efficiency (measured on the GPT-3-sized product: 192-wide tiles reach 0.92 / 0.85 of the 256x256
-// rate, 128x128 tiles about 0.7).
+// efficiency (measured on the GPT-3-sized product, per flop: 192-wide tiles reach about 0.93 of the
+// 256x256 rate, 128x128 tiles about 0.55).  All defaults use four waves over two 64-deep stages:
+// whole 128-byte lines per request for k-contiguous operands, half as many barriers as 32-deep stages.
 int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
   int v = g_variant;
   if (v == 0) {
     struct Cand { int v, bm, bn; double eff; };
-    const Cand cands[] = {{4, 256, 256, 1.0}, {5, 256, 192, 0.92}, {6, 192, 256, 0.85}, {3, 128, 128, 0.70}};
+    const Cand cands[] = {{1, 256, 256, 1.0}, {8, 256, 192, 0.93}, {9, 192, 256, 0.93}, {3, 128, 128, 0.55}};
     const long chunks = p.flow == OS ? 1 : p.S;
     double best = 0;
     for (const Cand &c : cands) {
@@ -195,9 +198,6 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
       const double cost = (double)rounds * c.bm * c.bn / c.eff;
       if (v == 0 || cost < best) { v = c.v; best = cost; }
     }
-    // 256x256: eight waves (two per SIMD) over 64-element stages measure 2-3 % faster than four waves
-    // over 32-element stages when a k-contiguous operand is involved (whole 128-byte lines per request)
-    if (v == 4 && p.flow != RS) v = 7;
   }
   switch (v) {
     case 1: return launch_bf16_tile<256, 256, 2, 2, 64, 2>(p, dev, stream);
@@ -207,6 +207,8 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
     case 5: return launch_bf16_tile<256, 192, 2, 2, 32, 4>(p, dev, stream);
     case 6: return launch_bf16_tile<192, 256, 2, 2, 32, 4>(p, dev, stream);
     case 7: return launch_bf16_tile<256, 256, 2, 4, 64, 2>(p, dev, stream);
+    case 8: return launch_bf16_tile<256, 192, 2, 2, 64, 2>(p, dev, stream);
+    case 9: return launch_bf16_tile<192, 256, 2, 2, 64, 2>(p, dev, stream);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }
@@ -313,7 +315,7 @@ MS_API long ms_query(int what) {
 }
 
 MS_API int ms_set_variant(int variant) {
-  if (variant < 0 || variant > 7) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  if (variant < 0 || variant > 9) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
   g_variant = variant;
   return MS_OK;
 }
