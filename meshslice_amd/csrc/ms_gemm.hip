@@ -9,6 +9,7 @@
 #include "meshslice_hip.h"
 
 #include "ms_gemm_bf16.hip.inc"
+#include "ms_gemm_bf16_big.hip.inc"
 #include "ms_gemm_f32.hip.inc"
 
 #define MS_API extern "C" __attribute__((visibility("default")))
@@ -32,6 +33,12 @@ MS_INSTANTIATE_RING(256, 256, 64, 2, 2, 4)
 MS_INSTANTIATE_RING(256, 192, 64, 2, 2, 2)
 MS_INSTANTIATE_RING(192, 256, 64, 2, 2, 2)
 #undef MS_INSTANTIATE_RING
+template __global__ void msk::gemm_bf16_big_kernel<true, false, true, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_big_kernel<true, false, false, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_big_kernel<true, false, true, true>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_big_kernel<true, false, false, true>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_big_kernel<true, true, false, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_big_kernel<false, false, false, false>(const msk::GemmArgs);
 
 namespace {
 
@@ -128,13 +135,19 @@ int validate(const Problem &p) {
   return MS_OK;
 }
 
-template <int BM, int BN, int BK_, int NS, int WGM, int WGN, bool AK, bool BKM, bool OBF, bool EPI>
+// BIG = false: gemm_bf16_ring_kernel<BM, BN, ...>; BIG = true: gemm_bf16_big_kernel (256x384x64, 2x2 waves, two stages)
+template <bool BIG, int BM, int BN, int BK_, int NS, int WGM, int WGN, bool AK, bool BKM, bool OBF, bool EPI>
 void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
-  msk::gemm_bf16_ring_kernel<BM, BN, BK_, NS, WGM, WGN, AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
+  if constexpr (!BIG) {
+    msk::gemm_bf16_ring_kernel<BM, BN, BK_, NS, WGM, WGN, AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
+  } else {
+    static_assert(BM == 256 && BN == 384 && BK_ == 64 && NS == 2 && WGM == 2 && WGN == 2, "the big-tile kernel has one shape");
+    msk::gemm_bf16_big_kernel<AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
+  }
 }
 
 // tile BM x BN, WGM x WGN waves, NS ring stages of BK_ k-elements
-template <int BM, int BN, int WGM, int WGN, int BK_, int NS>
+template <int BM, int BN, int WGM, int WGN, int BK_, int NS, bool BIG = false>
 int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
@@ -160,16 +173,16 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   const bool epi = p.act != 0 || p.res || p.row_sum || p.row_sumsq;
   if (p.flow == OS) {
     if (epi) {
-      if (obf) launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, true, true>(gd, bd, stream, g);
-      else launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, false, true>(gd, bd, stream, g);
+      if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, true, true>(gd, bd, stream, g);
+      else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, false, true>(gd, bd, stream, g);
     } else {
-      if (obf) launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, true, false>(gd, bd, stream, g);
-      else launch_one<BM, BN, BK_, NS, WGM, WGN, true, false, false, false>(gd, bd, stream, g);
+      if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, true, false>(gd, bd, stream, g);
+      else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, false, false>(gd, bd, stream, g);
     }
   } else if (p.flow == LS) {
-    launch_one<BM, BN, BK_, NS, WGM, WGN, true, true, false, false>(gd, bd, stream, g);
+    launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, true, false, false>(gd, bd, stream, g);
   } else {
-    launch_one<BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
+    launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
   }
   MS_HIP(hipGetLastError());
   return MS_OK;
@@ -179,6 +192,7 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
 //   1: 256x256, 4 waves, 2 x 64     2: 256x256, 8 waves, 4 x 32     3: 128x128, 4 waves, 2 x 64
 //   4: 256x256, 4 waves, 4 x 32     5: 256x192, 4 waves, 4 x 32     6: 192x256, 4 waves, 4 x 32
 //   7: 256x256, 8 waves, 2 x 64     8: 256x192, 4 waves, 2 x 64     9: 192x256, 4 waves, 2 x 64
+//  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel)
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
 // ceil(tiles / CUs) rounds of one tile per CU, so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized product, per flop: 192-wide tiles reach about 0.93 of the
@@ -209,6 +223,7 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
     case 7: return launch_bf16_tile<256, 256, 2, 4, 64, 2>(p, dev, stream);
     case 8: return launch_bf16_tile<256, 192, 2, 2, 64, 2>(p, dev, stream);
     case 9: return launch_bf16_tile<192, 256, 2, 2, 64, 2>(p, dev, stream);
+    case 10: return launch_bf16_tile<256, 384, 2, 2, 64, 2, true>(p, dev, stream);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }
@@ -315,7 +330,7 @@ MS_API long ms_query(int what) {
 }
 
 MS_API int ms_set_variant(int variant) {
-  if (variant < 0 || variant > 9) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  if (variant < 0 || variant > 10) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
   g_variant = variant;
   return MS_OK;
 }
