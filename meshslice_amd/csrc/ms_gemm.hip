@@ -119,6 +119,13 @@ int validate(const Problem &p) {
   if (a_cont % q || b_cont % q) return fail(MS_ERR_ARG, "%s: contiguous extents (%d, %d) must be multiples of %d", fn, a_cont, b_cont, q);
   if (p.lda < a_cont || p.ldb < b_cont || p.ldc < p.N) return fail(MS_ERR_ARG, "%s: leading dimension smaller than the row length", fn);
   if (p.lda % q || p.ldb % q) return fail(MS_ERR_ARG, "%s: operand leading dimensions must be multiples of %d", fn, q);
+  {
+    // the kernels address an operand slice with 32-bit byte offsets, the upper half reserved for "out of range"
+    const long long a_rows = p.flow == RS ? p.K : p.M, b_rows = p.flow == LS ? p.N : p.K;
+    const long long es = p.in_dtype == MS_DTYPE_BF16 ? 2 : 4;
+    if (a_rows * p.lda * es > 0x7FFFFFFFLL || b_rows * p.ldb * es > 0x7FFFFFFFLL)
+      return fail(MS_ERR_UNSUPPORTED, "%s: an operand slice spans 2 GiB or more", fn);
+  }
   const int qo = p.out_dtype == MS_DTYPE_BF16 ? 8 : 4;
   if (p.N % qo || p.ldc % qo) return fail(MS_ERR_ARG, "%s: output columns / leading dimension must be multiples of %d", fn, qo);
   if (p.act != MS_ACT_NONE && p.act != MS_ACT_GELU) return fail(MS_ERR_ARG, "%s: unknown activation %d", fn, p.act);
@@ -195,15 +202,17 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
 //  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel)
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
 // ceil(tiles / CUs) rounds of one tile per CU, so the estimate is rounds x tile area / relative tile
-// efficiency (measured on the GPT-3-sized product, per flop: 192-wide tiles reach about 0.93 of the
-// 256x256 rate, 128x128 tiles about 0.55).  All defaults use four waves over two 64-deep stages:
-// whole 128-byte lines per request for k-contiguous operands, half as many barriers as 32-deep stages.
+// efficiency (measured on the GPT-3-sized product, per flop, 256x256 = 1: the 256x384 tile reaches 1.06
+// with a k-contiguous A and 0.85 without, 192-wide tiles about 0.93, 128x128 tiles about 0.55).  The
+// ring-kernel defaults use four waves over two 64-deep stages: whole 128-byte lines per request for
+// k-contiguous operands, half as many barriers as 32-deep stages.
 int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
   int v = g_variant;
   if (v == 0) {
     struct Cand { int v, bm, bn; double eff; };
-    const Cand cands[] = {{1, 256, 256, 1.0}, {8, 256, 192, 0.93}, {9, 192, 256, 0.93}, {3, 128, 128, 0.55}};
+    const Cand cands[] = {{1, 256, 256, 1.0}, {10, 256, 384, p.flow == RS ? 0.85 : 1.06}, {8, 256, 192, 0.93},
+                          {9, 192, 256, 0.93}, {3, 128, 128, 0.55}};
     const long chunks = p.flow == OS ? 1 : p.S;
     double best = 0;
     for (const Cand &c : cands) {
