@@ -405,6 +405,16 @@ def test_fused_epilogue_gelu_residual_moments(variant, out_dtype):
     assert orc.rel_frobenius(host(s1b), host(plain).sum(1)) <= 1e-4
 
 
+def test_operand_span_of_2gib_is_rejected():
+    """32-bit byte offsets inside the kernels: an operand slice of 2 GiB or more is refused, not mis-addressed."""
+    lib = _lib.load()
+    a = torch.zeros((8, 8), dtype=torch.bfloat16, device="cuda")
+    pa, _ka = _lib.ptr_array([a.data_ptr()]); pc = ctypes.c_void_p(a.data_ptr())
+    big_ld = 1 << 20                       # 1024 rows x 2^20 elements x 2 bytes = 2 GiB
+    rc = lib.ms_gemm_os(pa, pa, 1, 1024, 8, 8, big_ld, 8, pc, 8, _lib.MS_DTYPE_BF16, _lib.MS_DTYPE_BF16, None)
+    assert rc == _lib.MS_ERR_UNSUPPORTED and b"2 GiB" in lib.ms_last_error()
+
+
 def test_fused_epilogue_rejections():
     a = torch.zeros((64, 64), dtype=torch.float32, device="cuda")
     with pytest.raises(_lib.MeshSliceError):                 # fp32 operands: no fused kernel
