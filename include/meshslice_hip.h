@@ -99,6 +99,18 @@ int ms_gemm_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int
                int m_slice, int n, int k,
                float *const *Y_chunks, int ldy, int in_dtype, void *stream);
 
+/* ms_gemm_ls / ms_gemm_rs with the chunks written in out_dtype (MS_DTYPE_F32 or MS_DTYPE_BF16; Y_chunks then
+ * points to buffers of that type, ldy in elements).  bf16 chunks are what the reference itself hands to its
+ * reduce-scatter for bf16 operands (the einsum result takes the operand dtype, TensorParallel.py:181-189,
+ * :203-212): half the bytes to write and to reduce, one rounding of the fp32 accumulator per chunk element.
+ * The fp32 entry points above keep the partial sums exact until after the reduction. */
+int ms_gemm_ls_ex(const void *A, int lda, const void *const *W_slices, int ldw, int S,
+                  int m, int n_slice, int k,
+                  void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream);
+int ms_gemm_rs_ex(const void *const *X_slices, int ldx, const void *W, int ldw, int S,
+                  int m_slice, int n, int k,
+                  void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream);
+
 /* Timing helpers (replace the wall-clock loop of CostModel.estimateMatmul, reference
  * CostModel.py:74-98): run the same call `warmup` times untimed, then `reps` times, each launch
  * bracketed by HIP events on `stream`; ms_out[r] receives the r-th launch's milliseconds.

@@ -29,7 +29,7 @@ LIB_PATH = os.path.join(_HERE, "libmeshslice_hip.so")
 
 EXPORTS = (
     "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
-    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_ls", "ms_gemm_rs",
+    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex",
     "ms_time_os", "ms_time_ls", "ms_time_rs",
 )
 
@@ -61,10 +61,12 @@ def _declare(lib):
     lib.ms_gemm_os.argtypes = os_args
     lib.ms_gemm_ls.argtypes = ls_args
     lib.ms_gemm_rs.argtypes = rs_args
+    lib.ms_gemm_ls_ex.argtypes = ls_args[:-1] + [c_int, c_vp]      # ..., in_dtype, out_dtype, stream
+    lib.ms_gemm_rs_ex.argtypes = rs_args[:-1] + [c_int, c_vp]
     lib.ms_time_os.argtypes = os_args + [c_int, c_int, fp]
     lib.ms_time_ls.argtypes = ls_args + [c_int, c_int, fp]
     lib.ms_time_rs.argtypes = rs_args + [c_int, c_int, fp]
-    for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_time_os", "ms_time_ls", "ms_time_rs"):
+    for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_time_os", "ms_time_ls", "ms_time_rs"):
         getattr(lib, n).restype = c_int
 
 

@@ -22,7 +22,9 @@
   template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, true, true>(const msk::GemmArgs);    \
   template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, false, false, true>(const msk::GemmArgs);   \
   template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, true, false, false>(const msk::GemmArgs);   \
-  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, false, false, false, false>(const msk::GemmArgs);
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, true, true, true, false>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, false, false, false, false>(const msk::GemmArgs); \
+  template __global__ void msk::gemm_bf16_ring_kernel<BM, BN, BK, NS, WGM, WGN, false, false, true, false>(const msk::GemmArgs);
 MS_INSTANTIATE_RING(256, 256, 64, 2, 2, 2)
 MS_INSTANTIATE_RING(256, 256, 32, 4, 2, 4)
 MS_INSTANTIATE_RING(128, 128, 64, 2, 2, 2)
@@ -38,7 +40,9 @@ template __global__ void msk::gemm_bf16_big_kernel<true, false, false, false>(co
 template __global__ void msk::gemm_bf16_big_kernel<true, false, true, true>(const msk::GemmArgs);
 template __global__ void msk::gemm_bf16_big_kernel<true, false, false, true>(const msk::GemmArgs);
 template __global__ void msk::gemm_bf16_big_kernel<true, true, false, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_big_kernel<true, true, true, false>(const msk::GemmArgs);
 template __global__ void msk::gemm_bf16_big_kernel<false, false, false, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_big_kernel<false, false, true, false>(const msk::GemmArgs);
 
 namespace {
 
@@ -187,9 +191,11 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
       else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, false, false>(gd, bd, stream, g);
     }
   } else if (p.flow == LS) {
-    launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, true, false, false>(gd, bd, stream, g);
+    if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, true, true, false>(gd, bd, stream, g);
+    else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, true, false, false>(gd, bd, stream, g);
   } else {
-    launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
+    if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, false, false, true, false>(gd, bd, stream, g);
+    else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
   }
   MS_HIP(hipGetLastError());
   return MS_OK;
@@ -313,12 +319,12 @@ Problem make_os(const void *const *A, const void *const *B, int S, int m, int n,
   return make_problem(OS, A, B, C, S, S, 1, S, m, n, k, lda, ldb, ldc, in_dtype, out_dtype);
 }
 Problem make_ls(const void *const *A, int lda, const void *const *W, int ldw, int S, int m, int n, int k,
-                float *const *Y, int ldy, int in_dtype) {
-  return make_problem(LS, A, W, (void *const *)Y, 1, S, S, S, m, n, k, lda, ldw, ldy, in_dtype, MS_DTYPE_F32);
+                void *const *Y, int ldy, int in_dtype, int out_dtype = MS_DTYPE_F32) {
+  return make_problem(LS, A, W, Y, 1, S, S, S, m, n, k, lda, ldw, ldy, in_dtype, out_dtype);
 }
 Problem make_rs(const void *const *X, int ldx, const void *const *W, int ldw, int S, int m, int n, int k,
-                float *const *Y, int ldy, int in_dtype) {
-  return make_problem(RS, X, W, (void *const *)Y, S, 1, S, S, m, n, k, ldx, ldw, ldy, in_dtype, MS_DTYPE_F32);
+                void *const *Y, int ldy, int in_dtype, int out_dtype = MS_DTYPE_F32) {
+  return make_problem(RS, X, W, Y, S, 1, S, S, m, n, k, ldx, ldw, ldy, in_dtype, out_dtype);
 }
 
 }  // namespace
@@ -364,13 +370,25 @@ MS_API int ms_gemm_os_fused(const void *const *A_slices, const void *const *B_sl
 MS_API int ms_gemm_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
                       float *const *Y_chunks, int ldy, int in_dtype, void *stream) {
   const void *a1[1] = {A};
-  return run(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, Y_chunks, ldy, in_dtype), stream);
+  return run(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, (void *const *)Y_chunks, ldy, in_dtype), stream);
 }
 
 MS_API int ms_gemm_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
                       float *const *Y_chunks, int ldy, int in_dtype, void *stream) {
   const void *w1[1] = {W};
-  return run(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype), stream);
+  return run(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, (void *const *)Y_chunks, ldy, in_dtype), stream);
+}
+
+MS_API int ms_gemm_ls_ex(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
+                         void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream) {
+  const void *a1[1] = {A};
+  return run(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, Y_chunks, ldy, in_dtype, out_dtype), stream);
+}
+
+MS_API int ms_gemm_rs_ex(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
+                         void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream) {
+  const void *w1[1] = {W};
+  return run(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype, out_dtype), stream);
 }
 
 MS_API int ms_time_os(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
@@ -383,11 +401,11 @@ MS_API int ms_time_os(const void *const *A_slices, const void *const *B_slices, 
 MS_API int ms_time_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
                       float *const *Y_chunks, int ldy, int in_dtype, void *stream, int warmup, int reps, float *ms_out) {
   const void *a1[1] = {A};
-  return timed(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, Y_chunks, ldy, in_dtype), stream, warmup, reps, ms_out);
+  return timed(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, (void *const *)Y_chunks, ldy, in_dtype), stream, warmup, reps, ms_out);
 }
 
 MS_API int ms_time_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
                       float *const *Y_chunks, int ldy, int in_dtype, void *stream, int warmup, int reps, float *ms_out) {
   const void *w1[1] = {W};
-  return timed(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype), stream, warmup, reps, ms_out);
+  return timed(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, (void *const *)Y_chunks, ldy, in_dtype), stream, warmup, reps, ms_out);
 }

@@ -97,46 +97,62 @@ def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
     return out
 
 
+def _chunk_dtype(out, out_dtype):
+    """dtype of the LS / RS chunks: that of ``out`` if given, else ``out_dtype``, else fp32."""
+    if out is not None and len(out) > 0:
+        if out_dtype is not None and out[0].dtype != out_dtype:
+            raise ValueError("out_dtype contradicts the dtype of out")
+        return out[0].dtype
+    dt = torch.float32 if out_dtype is None else out_dtype
+    if dt not in (torch.float32, torch.bfloat16):
+        raise ValueError("chunks are fp32 or bf16")
+    return dt
+
+
 def gemm_ls(A: torch.Tensor, W_slices: Sequence[torch.Tensor],
-            out: Optional[List[torch.Tensor]] = None) -> List[torch.Tensor]:
-    """``Y_s = A @ W_s^T`` (fp32 chunks), W_s stored ``[n_slice, k]``."""
+            out: Optional[List[torch.Tensor]] = None, out_dtype: Optional[torch.dtype] = None) -> List[torch.Tensor]:
+    """``Y_s = A @ W_s^T``, W_s stored ``[n_slice, k]``.  Chunks are fp32 by default (exact partial sums for
+    the reduce-scatter); ``out_dtype=torch.bfloat16`` gives what the reference's einsum returns for bf16
+    operands (TensorParallel.py:181-189): one rounding of the fp32 accumulator, half the bytes."""
     _check2d(A, "A"); w0 = _same(W_slices, "W_slices")
     if A.shape[1] != w0.shape[1] or A.dtype != w0.dtype:
         raise ValueError(f"shapes do not contract: {tuple(A.shape)} @ {tuple(w0.shape)}^T")
     m, k = A.shape; ns = w0.shape[0]; S = len(W_slices)
+    dt = _chunk_dtype(out, out_dtype)
     if out is None:
-        buf = torch.empty((S, m, ns), dtype=torch.float32, device=A.device)
+        buf = torch.empty((S, m, ns), dtype=dt, device=A.device)
         out = [buf[s] for s in range(S)]
     o0 = _same(out, "out")
-    if len(out) != S or tuple(o0.shape) != (m, ns) or o0.dtype != torch.float32:
-        raise ValueError("out must be S fp32 chunks of shape [m, n_slice]")
+    if len(out) != S or tuple(o0.shape) != (m, ns) or o0.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("out must be S fp32 or bf16 chunks of shape [m, n_slice]")
     pw, _kw = _lib.ptr_array([t.data_ptr() for t in W_slices])
     py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
     with torch.cuda.device(A.device):
-        rc = _lib.load().ms_gemm_ls(ctypes.c_void_p(A.data_ptr()), A.stride(0), pw, w0.stride(0), S, m, ns, k,
-                                    py, o0.stride(0), _dt(A), _stream())
+        rc = _lib.load().ms_gemm_ls_ex(ctypes.c_void_p(A.data_ptr()), A.stride(0), pw, w0.stride(0), S, m, ns, k,
+                                       py, o0.stride(0), _dt(A), _dt(o0), _stream())
     _lib.check(rc)
     return list(out)
 
 
 def gemm_rs(X_slices: Sequence[torch.Tensor], W: torch.Tensor,
-            out: Optional[List[torch.Tensor]] = None) -> List[torch.Tensor]:
-    """``Y_s = X_s^T @ W`` (fp32 chunks), X_s stored ``[k, m_slice]``."""
+            out: Optional[List[torch.Tensor]] = None, out_dtype: Optional[torch.dtype] = None) -> List[torch.Tensor]:
+    """``Y_s = X_s^T @ W``, X_s stored ``[k, m_slice]``; chunks fp32 by default, bf16 on request (see gemm_ls)."""
     _check2d(W, "W"); x0 = _same(X_slices, "X_slices")
     if x0.shape[0] != W.shape[0] or x0.dtype != W.dtype:
         raise ValueError(f"shapes do not contract: {tuple(x0.shape)}^T @ {tuple(W.shape)}")
     k, ms = x0.shape; n = W.shape[1]; S = len(X_slices)
+    dt = _chunk_dtype(out, out_dtype)
     if out is None:
-        buf = torch.empty((S, ms, n), dtype=torch.float32, device=W.device)
+        buf = torch.empty((S, ms, n), dtype=dt, device=W.device)
         out = [buf[s] for s in range(S)]
     o0 = _same(out, "out")
-    if len(out) != S or tuple(o0.shape) != (ms, n) or o0.dtype != torch.float32:
-        raise ValueError("out must be S fp32 chunks of shape [m_slice, n]")
+    if len(out) != S or tuple(o0.shape) != (ms, n) or o0.dtype not in (torch.float32, torch.bfloat16):
+        raise ValueError("out must be S fp32 or bf16 chunks of shape [m_slice, n]")
     px, _kx = _lib.ptr_array([t.data_ptr() for t in X_slices])
     py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
     with torch.cuda.device(W.device):
-        rc = _lib.load().ms_gemm_rs(px, x0.stride(0), ctypes.c_void_p(W.data_ptr()), W.stride(0), S, ms, n, k,
-                                    py, o0.stride(0), _dt(W), _stream())
+        rc = _lib.load().ms_gemm_rs_ex(px, x0.stride(0), ctypes.c_void_p(W.data_ptr()), W.stride(0), S, ms, n, k,
+                                       py, o0.stride(0), _dt(W), _dt(o0), _stream())
     _lib.check(rc)
     return list(out)
 

@@ -180,6 +180,40 @@ def test_bf16_output_is_one_rounding_of_the_fp32_accumulator():
     assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize("variant", [0, 1, 3, 5, 8, 10])
+@pytest.mark.parametrize("flow", ["ls", "rs"])
+@pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
+def test_bf16_chunks_are_one_rounding_of_the_fp32_chunks(flow, variant, in_dtype):
+    """ms_gemm_ls_ex / ms_gemm_rs_ex with bf16 chunks (what the reference's einsum hands to its reduce-scatter):
+    every chunk equals the round-to-nearest-even of the fp32 chunk of the same call, bit for bit, also on
+    ragged shapes, and nothing is written outside a strided chunk."""
+    if in_dtype == torch.float32 and variant != 0:
+        pytest.skip("kernel variants are bf16 kernels")
+    _lib.check(_lib.load().ms_set_variant(variant))
+    for (m, n, k, S) in [(512, 768, 256, 3), (264, 520, 72, 2), (1000, 776, 328, 2)]:
+        ops = _rand_case(flow, m, n, k, S, seed=17 + variant, dtype=in_dtype)
+        if flow == "ls":
+            A, W = ops
+            a = dev(A, in_dtype); w = [dev(x, in_dtype) for x in W]
+            y32 = ms.gemm_ls(a, w)
+            pad = torch.zeros((S, m, n + 8), dtype=torch.bfloat16, device="cuda")
+            y16 = ms.gemm_ls(a, w, out=[pad[s][:, :n] for s in range(S)])
+        else:
+            X, W = ops
+            x = [dev(t, in_dtype) for t in X]; w = dev(W, in_dtype)
+            y32 = ms.gemm_rs(x, w)
+            pad = torch.zeros((S, m, n + 8), dtype=torch.bfloat16, device="cuda")
+            y16 = ms.gemm_rs(x, w, out=[pad[s][:, :n] for s in range(S)])
+        for c32, c16 in zip(y32, y16):
+            assert c16.dtype == torch.bfloat16
+            want = orc.bf16_bits(c32.cpu().numpy())
+            got = c16.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+            assert np.array_equal(got, want)
+        assert float(pad[:, :, n:].abs().max()) == 0.0
+    fresh = ms.gemm_ls(a, w, out_dtype=torch.bfloat16) if flow == "ls" else ms.gemm_rs(x, w, out_dtype=torch.bfloat16)
+    assert all(torch.equal(f, c) for f, c in zip(fresh, y16))
+
+
 def test_strided_operands_and_outputs():
     """Leading dimensions larger than the row length (slices that are views of a bigger buffer)."""
     rng = np.random.default_rng(5)
