@@ -128,6 +128,34 @@ int ms_time_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int
                float *const *Y_chunks, int ldy, int in_dtype, void *stream,
                int warmup, int reps, float *ms_out);
 
+/* Block-cyclic slices of a shard, all S of them in one pass over it:
+ *     axis 1:  dst_slices[s][r, (b / S) * B + e] = src[r, b * B + e]   for column blocks b with b % S == s
+ *     axis 0:  dst_slices[s][(b / S) * B + e, c] = src[b * B + e, c]   for row blocks b with b % S == s
+ * Replaces the reshape to (.., L/(S*B), S, B) and the dynamic_slice_in_dim along the S axis with which a
+ * mesh device cuts slice s out of its shard before the all-gather (TensorParallel.py:155-158, :177-178,
+ * :198-199).  src is [rows, cols] (ld_src); slice s is [rows, cols / S] (axis 1) or [rows / S, cols]
+ * (axis 0) with leading dimension ld_dst, so a slice can be written straight into its place in a larger
+ * gathered buffer.  The sliced extent must be a multiple of S * B.  dtype only sets the element size.
+ * Pointers need the alignment of one element; 16-byte aligned pointers, row lengths and leading
+ * dimensions (and B elements a multiple of 16 bytes for axis 1) select the 16-byte kernels. */
+int ms_pack_slices(const void *src, int ld_src, int rows, int cols, int axis, int S, int B,
+                   void *const *dst_slices, int ld_dst, int dtype, void *stream);
+
+/* The inverse placement, for a device's output shard, with the sum a reduce-scatter takes on the way:
+ *     axis 1:  out[r, (h * S + s) * B + e] = sum_{p<P} chunks[p * S + s][row_off + r, col_off + h * B + e]
+ *     axis 0:  out[(h * S + s) * B + e, c] = sum_{p<P} chunks[p * S + s][row_off + h * B + e, col_off + c]
+ * Replaces psum_scatter of partial chunk s (the sum over the P peers and the choice of this device's
+ * window, TensorParallel.py:182,188,204,210), the dynamic_update_slice_in_dim that puts the result at
+ * slice position s of the (.., S, B) view of the output shard (:184,190,206,211) and the final reshape
+ * (:193,:214).  out is [rows, cols] (ld_out) in out_dtype; each chunk has leading dimension ld_chunk and
+ * element type in_dtype, and (row_off, col_off) is the corner of the window of every chunk that this
+ * device keeps, [rows, cols / S] (axis 1) or [rows / S, cols] (axis 0).  With P == 1 (chunks already
+ * reduced, as after a real reduce-scatter) it is a pure placement.  The sum runs in fp32 in peer order
+ * and is rounded once (round-to-nearest-even) to out_dtype.  P * S <= 64. */
+int ms_unpack_chunks(const void *const *chunks, int P, int S, int ld_chunk, int row_off, int col_off,
+                     int rows, int cols, int axis, int B, void *out, int ld_out,
+                     int in_dtype, int out_dtype, void *stream);
+
 /* Tuning knob for experiments: selects the bf16 kernel variant used by later calls on this
  * thread (0 = library default).  Unknown ids are rejected with MS_ERR_ARG. */
 int ms_set_variant(int variant);

@@ -9,7 +9,9 @@ by having one GPU and no tracing compiler:
   sharded ``P(row, col)``, and returns the GLOBAL result; it runs every mesh device's body in turn;
 * ``.device(i, j)`` runs ONE device's body and returns what that device produces before any
   cross-device reduction: its output block (OS) or its S fp32 partial chunks (LS / RS);
-* all_gather / psum_scatter are host-side index arithmetic over the list of shards;
+* all_gather / psum_scatter move data between the emulated devices' buffers on the one GPU: the
+  block-cyclic slicing, the placement of gathered slices and the reduce + interleave of the chunks run
+  in the layout kernels of libmeshslice_hip.so (slice_layout.py), not in torch indexing;
 * the local contraction accumulates in fp32 over all slices and rounds once (the reference carries
   the running sum in the input dtype, :167);
 * the sliced OS body rejects ``K == 1``: the reference adds slice 0 twice in that case (:163,:172);
@@ -22,7 +24,7 @@ from typing import Callable, List, Sequence
 
 import torch
 
-from . import local_gemm
+from . import local_gemm, slice_layout
 from .mesh import Mesh, PartitionSpec as P  # noqa: F401  (re-exported like the reference's imports)
 
 
@@ -50,24 +52,44 @@ def _need(v: int, d: int, what: str) -> None:
         raise ValueError(f"{what} = {v} is not a multiple of {d}")
 
 
-def _slice_cols(block: torch.Tensor, k: int, K: int, B: int) -> torch.Tensor:
-    """Slice k of the column view (rows, cols/(K*B), K, B) -> (rows, cols/K)   (reference :155,157)."""
-    r, c = block.shape
-    _need(c, K * B, "sliced extent")
-    return block.reshape(r, c // (K * B), K, B)[:, :, k, :].reshape(r, c // K)
-
-
-def _slice_rows(block: torch.Tensor, k: int, K: int, B: int) -> torch.Tensor:
-    """Slice k of the row view (rows/(K*B), K, B, cols) -> (rows/K, cols)   (reference :156,158)."""
-    r, c = block.shape
-    _need(r, K * B, "sliced extent")
-    return block.reshape(r // (K * B), K, B, c)[:, k, :, :].reshape(r // K, c)
+def _own(block: torch.Tensor) -> torch.Tensor:
+    """A device's shard as the kernels can address it: the view itself when its first element and its rows
+    are 16-byte aligned (a real device's shard is its own buffer), else a contiguous copy."""
+    if block.stride(1) == 1 and block.data_ptr() % 16 == 0 and (block.stride(0) * block.element_size()) % 16 == 0:
+        return block
+    return block.contiguous()
 
 
 def _gather(parts: Sequence[torch.Tensor], axis: int) -> torch.Tensor:
-    """tiled all_gather as the receiving device sees it: peers' parts concatenated in axis order,
-    materialised contiguous in HBM (what a real all-gather delivers)."""
+    """tiled all_gather of whole shards as the receiving device sees it: peers' parts concatenated in axis
+    order, materialised contiguous in HBM (what a real all-gather delivers)."""
     return torch.cat(list(parts), dim=axis).contiguous()
+
+
+def _gather_col_slices(peers: Sequence[torch.Tensor], K: int, B: int) -> List[torch.Tensor]:
+    """The K gathered column slices ``[rows, len(peers) * cols / K]``: every peer cuts its shard's columns into
+    K block-cyclic slices (reference :155,157,198-199) and slice k of peer p lands at column block p of
+    gathered slice k (all_gather over the peers' axis, tiled along the columns).  One kernel per peer writes
+    its K slices straight into their places; there is no separate concatenation."""
+    r, c = peers[0].shape
+    _need(c, K * B, "sliced extent")
+    w = c // K
+    buf = torch.empty((K, r, len(peers) * w), dtype=peers[0].dtype, device=peers[0].device)
+    for p, blk in enumerate(peers):
+        slice_layout.pack_slices(blk, K, B, 1, out=[buf[k][:, p * w:(p + 1) * w] for k in range(K)])
+    return [buf[k] for k in range(K)]
+
+
+def _gather_row_slices(peers: Sequence[torch.Tensor], K: int, B: int) -> List[torch.Tensor]:
+    """The K gathered row slices ``[len(peers) * rows / K, cols]`` (reference :156,158,177-178), peer p's part
+    of slice k at row block p."""
+    r, c = peers[0].shape
+    _need(r, K * B, "sliced extent")
+    h = r // K
+    buf = torch.empty((K, len(peers) * h, c), dtype=peers[0].dtype, device=peers[0].device)
+    for p, blk in enumerate(peers):
+        slice_layout.pack_slices(blk, K, B, 0, out=[buf[k][p * h:(p + 1) * h] for k in range(K)])
+    return [buf[k] for k in range(K)]
 
 
 # ------------------------------------------------------------------------------------------------
@@ -85,13 +107,13 @@ def Collective_OS(X, W, i, j, R, C, K, B):
 def Collective_LS(X, W, i, j, R, C, K, B):
     """reference :24-27: gather W over row; partial product X_ij @ Wj^T (input of psum_scatter)."""
     Wj = _gather([W[ii][j] for ii in range(R)], 0)
-    return local_gemm.gemm_ls(X[i][j].contiguous(), [Wj])
+    return local_gemm.gemm_ls(_own(X[i][j]), [Wj])
 
 
 def Collective_RS(X, W, i, j, R, C, K, B):
     """reference :29-32: gather X over col; partial product Xi^T @ W_ij (input of psum_scatter)."""
     Xi = _gather([X[i][jj] for jj in range(C)], 1)
-    return local_gemm.gemm_rs([Xi], W[i][j].contiguous())
+    return local_gemm.gemm_rs([Xi], _own(W[i][j]))
 
 
 def MeshFlow_OS(X, W, i, j, R, C, K, B):
@@ -99,53 +121,42 @@ def MeshFlow_OS(X, W, i, j, R, C, K, B):
     if K == 1:
         raise ValueError("the sliced OS body is undefined for K == 1 (the reference adds slice 0 twice); "
                          "use algorithm='collective' for the unsliced product")
-    A_slices = [_gather([_slice_cols(X[i][jj], k, K, B) for jj in range(C)], 1) for k in range(K)]
-    B_slices = [_gather([_slice_rows(W[ii][j], k, K, B) for ii in range(R)], 0) for k in range(K)]
+    A_slices = _gather_col_slices([X[i][jj] for jj in range(C)], K, B)
+    B_slices = _gather_row_slices([W[ii][j] for ii in range(R)], K, B)
     return local_gemm.gemm_os(A_slices, B_slices)
 
 
 def MeshFlow_LS(X, W, i, j, R, C, K, B):
     """reference :174-193: K gathered row slices of W; K fp32 partial chunks X_ij @ W_k^T."""
-    W_slices = [_gather([_slice_rows(W[ii][j], k, K, B) for ii in range(R)], 0) for k in range(K)]
-    return local_gemm.gemm_ls(X[i][j].contiguous(), W_slices)
+    W_slices = _gather_row_slices([W[ii][j] for ii in range(R)], K, B)
+    return local_gemm.gemm_ls(_own(X[i][j]), W_slices)
 
 
 def MeshFlow_RS(X, W, i, j, R, C, K, B):
     """reference :195-214: K gathered column slices of X; K fp32 partial chunks X_k^T @ W_ij."""
-    X_slices = [_gather([_slice_cols(X[i][jj], k, K, B) for jj in range(C)], 1) for k in range(K)]
-    return local_gemm.gemm_rs(X_slices, W[i][j].contiguous())
+    X_slices = _gather_col_slices([X[i][jj] for jj in range(C)], K, B)
+    return local_gemm.gemm_rs(X_slices, _own(W[i][j]))
 
 
 # ------------------------------------------------------------------------------------------------
 # mesh completion: what psum_scatter + the (.., K, B) interleave do with the partial chunks
 # ------------------------------------------------------------------------------------------------
 
-def _finish_ls(chunks_by_col, j, C, K, B, dtype):
-    """psum over the mesh row, keep device column j's blocks, interleave (reference :182-193)."""
-    m, os_ = chunks_by_col[0][0].shape
-    nb = os_ // B                       # B-wide blocks in one gathered slice
-    _need(nb, C, "blocks per slice")
-    out = torch.empty((m, nb // C, K, B), dtype=torch.float32, device=chunks_by_col[0][0].device)
-    for k in range(K):
-        tot = chunks_by_col[0][k].clone()
-        for jj in range(1, C):
-            tot += chunks_by_col[jj][k]
-        out[:, :, k, :] = tot.reshape(m, nb, B)[:, j * (nb // C):(j + 1) * (nb // C), :]
-    return out.reshape(m, -1).to(dtype)
-
-
-def _finish_rs(chunks_by_row, i, R, K, B, dtype):
-    """psum over the mesh column, keep device row i's blocks, interleave (reference :204-214)."""
-    ns, n = chunks_by_row[0][0].shape
-    nb = ns // B
-    _need(nb, R, "blocks per slice")
-    out = torch.empty((nb // R, K, B, n), dtype=torch.float32, device=chunks_by_row[0][0].device)
-    for k in range(K):
-        tot = chunks_by_row[0][k].clone()
-        for ii in range(1, R):
-            tot += chunks_by_row[ii][k]
-        out[:, k, :, :] = tot.reshape(nb, B, n)[i * (nb // R):(i + 1) * (nb // R), :, :]
-    return out.reshape(-1, n).to(dtype)
+def _finish(chunks_by_peer, me, axis, B, dtype):
+    """psum_scatter over the peers (device ``me`` of them keeps its window of every summed chunk) and the
+    interleave of the K windows into the output shard: reference :182-193 (LS: peers = the mesh row,
+    axis 1) and :204-214 (RS: peers = the mesh column, axis 0).  One kernel; the sum is fp32 in peer
+    order with one rounding to ``dtype``."""
+    P, K = len(chunks_by_peer), len(chunks_by_peer[0])
+    if P * K > 64:  # more pointers than one launch takes: sum the peers first, then place
+        tot = []
+        for k in range(K):
+            t = chunks_by_peer[0][k].clone()
+            for p in range(1, P):
+                t += chunks_by_peer[p][k]
+            tot.append(t)
+        chunks_by_peer = [tot]
+    return slice_layout.unpack_chunks(chunks_by_peer, B, axis, window=me, parts=P, out_dtype=dtype)
 
 
 class ShardedMatmul:
@@ -213,7 +224,7 @@ class ShardedMatmul:
                     tot = sum(c[0] for c in chunks)
                     rows.append(tot.to(X.dtype))
                 else:
-                    rows.append(torch.cat([_finish_ls(chunks, j, C, K, B, X.dtype) for j in range(C)], dim=1))
+                    rows.append(torch.cat([_finish(chunks, j, 1, B, X.dtype) for j in range(C)], dim=1))
             return torch.cat(rows, dim=0)
         cols = []
         for j in range(C):
@@ -221,7 +232,7 @@ class ShardedMatmul:
             if not self.sliced:
                 cols.append(sum(c[0] for c in chunks).to(X.dtype))
             else:
-                cols.append(torch.cat([_finish_rs(chunks, i, R, K, B, X.dtype) for i in range(R)], dim=0))
+                cols.append(torch.cat([_finish(chunks, i, 0, B, X.dtype) for i in range(R)], dim=0))
         return torch.cat(cols, dim=1)
 
 

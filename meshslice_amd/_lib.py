@@ -31,6 +31,7 @@ EXPORTS = (
     "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
     "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex",
     "ms_time_os", "ms_time_ls", "ms_time_rs",
+    "ms_pack_slices", "ms_unpack_chunks",
 )
 
 _lock = threading.Lock()
@@ -66,6 +67,12 @@ def _declare(lib):
     lib.ms_time_os.argtypes = os_args + [c_int, c_int, fp]
     lib.ms_time_ls.argtypes = ls_args + [c_int, c_int, fp]
     lib.ms_time_rs.argtypes = rs_args + [c_int, c_int, fp]
+    # src, ld_src, rows, cols, axis, S, B, dst_slices, ld_dst, dtype, stream
+    lib.ms_pack_slices.argtypes = [c_vp, c_int, c_int, c_int, c_int, c_int, c_int, vpp, c_int, c_int, c_vp]
+    lib.ms_pack_slices.restype = c_int
+    # chunks, P, S, ld_chunk, row_off, col_off, rows, cols, axis, B, out, ld_out, in_dtype, out_dtype, stream
+    lib.ms_unpack_chunks.argtypes = [vpp, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_vp, c_int, c_int, c_int, c_vp]
+    lib.ms_unpack_chunks.restype = c_int
     for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_time_os", "ms_time_ls", "ms_time_rs"):
         getattr(lib, n).restype = c_int
 

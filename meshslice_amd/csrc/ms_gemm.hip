@@ -6,13 +6,11 @@
 #include <cstdio>
 #include <cstring>
 
-#include "meshslice_hip.h"
+#include "ms_common.hip.inc"
 
 #include "ms_gemm_bf16.hip.inc"
 #include "ms_gemm_bf16_big.hip.inc"
 #include "ms_gemm_f32.hip.inc"
-
-#define MS_API extern "C" __attribute__((visibility("default")))
 
 // Every kernel variant is instantiated explicitly: with implicit instantiation alone the host
 // compiler leaves some of the launch stubs undefined.
@@ -45,11 +43,10 @@ template __global__ void msk::gemm_bf16_big_kernel<false, false, false, false>(c
 template __global__ void msk::gemm_bf16_big_kernel<false, false, true, false>(const msk::GemmArgs);
 
 namespace {
-
 thread_local char g_err[512] = "";
-thread_local int g_variant = 0;
+}
 
-int fail(int code, const char *fmt, ...) {
+int msi::fail(int code, const char *fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
   vsnprintf(g_err, sizeof(g_err), fmt, ap);
@@ -57,11 +54,11 @@ int fail(int code, const char *fmt, ...) {
   return code;
 }
 
-#define MS_HIP(call)                                                                        \
-  do {                                                                                      \
-    hipError_t e_ = (call);                                                                 \
-    if (e_ != hipSuccess) return fail(MS_ERR_HIP, "%s failed: %s", #call, hipGetErrorString(e_)); \
-  } while (0)
+namespace {
+
+thread_local int g_variant = 0;
+
+using msi::fail;
 
 struct DevInfo {
   int valid, cus, clock_khz, gfx950, lds;

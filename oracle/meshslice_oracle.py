@@ -249,6 +249,57 @@ def assemble_rs(chunks_by_row, R, C, i, S, B):
 
 
 # --------------------------------------------------------------------------------------
+# the layout steps either side of the contraction, statement by statement
+# --------------------------------------------------------------------------------------
+
+def pack_slices(block: np.ndarray, S: int, B: int, axis: int):
+    """The S slices a device cuts out of its shard before the all-gathers: the reshape to
+    ``(rows, cols/(S*B), S, B)`` (axis 1, TensorParallel.py:155,157,198-199) or
+    ``(rows/(S*B), S, B, cols)`` (axis 0, :156,158,177-178) followed by ``dynamic_slice_in_dim(.., k, 1)``
+    along the S axis and the flattening the einsum subscripts imply."""
+    r, c = block.shape
+    if S < 1 or B < 1 or (c if axis == 1 else r) % (S * B):
+        raise ValueError("sliced extent is not a multiple of S*B")
+    out = []
+    for k in range(S):
+        if axis == 1:
+            v = block.reshape(r, c // (S * B), S, B)
+            out.append(np.ascontiguousarray(_dyn_slice(v, k, 1, 2)).reshape(r, c // S))
+        else:
+            v = block.reshape(r // (S * B), S, B, c)
+            out.append(np.ascontiguousarray(_dyn_slice(v, k, 1, 1)).reshape(r // S, c))
+    return out
+
+
+def unpack_chunks(chunks_by_peer, B: int, axis: int, window: int = 0, parts: int = 1, out_dtype=np.float32):
+    """A device's output shard from its peers' partial chunks: tiled ``psum_scatter`` of chunk k along
+    ``axis`` over ``parts`` devices, of which this one is number ``window`` (TensorParallel.py:182,188,
+    204,210: sum over the peers in fp32, in peer order; keep the window), ``dynamic_update_slice_in_dim``
+    at position k of the zero-initialised ``(.., S, B)`` view (:179,184,190 / :200,206,211), final reshape
+    (:193,:214).  ``out_dtype`` np.float32, or "bf16" for the fp32 sum rounded once to bf16 (returned as
+    float32 values)."""
+    S = len(chunks_by_peer[0])
+    cr, cc = chunks_by_peer[0][0].shape
+    cut = cc if axis == 1 else cr
+    if cut % parts or (cut // parts) % B:
+        raise ValueError("chunk does not split into windows of whole blocks")
+    keep = cut // parts
+    nb = keep // B
+    Y = np.zeros((cr, nb, S, B), np.float32) if axis == 1 else np.zeros((nb, S, B, cc), np.float32)
+    for k in range(S):
+        tot = np.array(chunks_by_peer[0][k], dtype=np.float32)
+        for peer in chunks_by_peer[1:]:
+            tot = tot + np.asarray(peer[k], dtype=np.float32)
+        mine = _dyn_slice(tot, window * keep, keep, axis)
+        if axis == 1:
+            Y[:, :, k:k + 1, :] = mine.reshape(cr, nb, 1, B)
+        else:
+            Y[:, k:k + 1, :, :] = mine.reshape(nb, 1, B, cc)
+    Y = Y.reshape(cr, keep * S) if axis == 1 else Y.reshape(keep * S, cc)
+    return bf16_round(Y) if out_dtype == "bf16" else Y
+
+
+# --------------------------------------------------------------------------------------
 # literal whole-mesh emulation of the reference bodies
 # --------------------------------------------------------------------------------------
 

@@ -48,40 +48,21 @@ def test_cpu_tensors_are_rejected_not_computed():
         TP.SPMD(mesh, "collective").OS()(torch.zeros(16, 16), torch.zeros(16, 16))
 
 
-# ---------------------------------------------------------------- mesh plumbing vs oracle
-@pytest.mark.parametrize("R,C,K,B", [(2, 2, 2, 2), (4, 2, 8, 8), (2, 4, 4, 8)])
-def test_slice_and_gather_match_closed_form(R, C, K, B):
-    L = R * C * K * B * 2
-    G = torch.arange(24 * L, dtype=torch.float32).reshape(24, L)
-    Xs = TP._shards(G, 4, C)
-    for k in range(K):
-        got = TP._gather([TP._slice_cols(Xs[1][jj], k, K, B) for jj in range(C)], 1)
-        want = G[6:12][:, torch.from_numpy(orc.sel(L, K, B, k))]
-        assert torch.equal(got, want)
-    Gt = G.t().contiguous()
-    Ws = TP._shards(Gt, R, 4)
-    for k in range(K):
-        got = TP._gather([TP._slice_rows(Ws[ii][2], k, K, B) for ii in range(R)], 0)
-        want = Gt[:, 12:18][torch.from_numpy(orc.sel(L, K, B, k)), :]
-        assert torch.equal(got, want)
-
-
-@pytest.mark.parametrize("R,C,S,B", [(2, 2, 2, 2), (4, 2, 4, 8), (2, 4, 2, 8)])
-def test_chunk_assembly_matches_oracle(R, C, S, B):
-    rng = np.random.default_rng(11)
-    O = R * C * S * B * 2
-    m = 6
-    chunks = [[rng.integers(-5, 6, (m, O // S)).astype(np.float32) for _ in range(S)] for _ in range(C)]
-    tch = [[torch.from_numpy(c) for c in row] for row in chunks]
-    for j in range(C):
-        got = TP._finish_ls(tch, j, C, S, B, torch.float32).numpy()
-        assert np.array_equal(got, orc.assemble_ls(chunks, R, C, j, S, B))
-    n = 5
-    chunks = [[rng.integers(-5, 6, (O // S, n)).astype(np.float32) for _ in range(S)] for _ in range(R)]
-    tch = [[torch.from_numpy(c) for c in row] for row in chunks]
-    for i in range(R):
-        got = TP._finish_rs(tch, i, R, S, B, torch.float32).numpy()
-        assert np.array_equal(got, orc.assemble_rs(chunks, R, C, i, S, B))
+# ---------------------------------------------------------------- mesh plumbing has no CPU path either
+def test_slicing_gathering_and_chunk_assembly_reject_cpu_tensors():
+    """The block-cyclic slicing, the gather placement and the reduce + interleave of the chunks run in HIP
+    kernels; on CPU tensors they raise instead of computing (their parity tests are GPU tests)."""
+    G = torch.arange(24 * 64, dtype=torch.float32).reshape(24, 64)
+    Xs = TP._shards(G, 4, 2)
+    assert Xs[1][1].shape == (6, 32) and Xs[1][1].data_ptr() == G[6:12, 32:].data_ptr()      # views, no copies
+    with pytest.raises(_lib.MeshSliceError):
+        TP._gather_col_slices([Xs[1][0], Xs[1][1]], 2, 8)
+    with pytest.raises(_lib.MeshSliceError):
+        TP._gather_row_slices([G[:16], G[:16]], 2, 8)
+    with pytest.raises(_lib.MeshSliceError):
+        TP._finish([[G, G], [G, G]], 0, 1, 8, torch.float32)
+    with pytest.raises(ValueError):
+        TP._gather_col_slices([Xs[1][0]], 3, 8)          # 32 columns are not a multiple of 3 * 8
 
 
 def test_spmd_surface_and_shape_errors():

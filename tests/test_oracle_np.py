@@ -44,6 +44,49 @@ def test_sel_rejects_bad_shapes():
         orc.sel(64, 4, 8, 4)
 
 
+# ---------------------------------------------------------------- layout steps
+
+@pytest.mark.parametrize("r,c,S,B", [(16, 32, 2, 2), (24, 64, 4, 8), (48, 96, 3, 8), (40, 120, 5, 4), (8, 16, 1, 8)])
+def test_pack_slices_matches_the_index_rule_and_brute_force(r, c, S, B):
+    """The literal reshape + dynamic_slice equals plain indexing with the closed-form rule, and with the
+    loop enumeration of the (.., S, B) view; the slices partition the shard."""
+    rng = np.random.default_rng(r * c + S)
+    blk = rng.integers(0, 1 << 30, size=(r, c)).astype(np.int64)
+    if c % (S * B) == 0:
+        sl = orc.pack_slices(blk, S, B, 1)
+        for k in range(S):
+            assert np.array_equal(sl[k], blk[:, orc.sel(c, S, B, k)])
+            assert np.array_equal(sl[k], blk[:, _sel_bruteforce(c, S, B, k)])
+        assert sorted(np.concatenate([x.ravel() for x in sl]).tolist()) == sorted(blk.ravel().tolist())
+    if r % (S * B) == 0:
+        sl = orc.pack_slices(blk, S, B, 0)
+        for k in range(S):
+            assert np.array_equal(sl[k], blk[orc.sel(r, S, B, k), :])
+            assert np.array_equal(sl[k], blk[_sel_bruteforce(r, S, B, k), :])
+
+
+@pytest.mark.parametrize("axis", [0, 1])
+@pytest.mark.parametrize("S,B,parts", [(2, 2, 2), (4, 8, 2), (3, 8, 1), (8, 8, 4)])
+def test_unpack_chunks_inverts_pack_and_matches_assembly(S, B, parts, axis):
+    """unpack(pack(x)) == x (one peer, one window); with several peers and windows it equals the closed-form
+    assembly (assemble_ls / assemble_rs), which the literal whole-mesh emulation pins elsewhere."""
+    rng = np.random.default_rng(S * 100 + B * 10 + parts + axis)
+    L = S * B * parts * 3
+    shape = (24, L) if axis == 1 else (L, 24)
+    x = rng.standard_normal(shape).astype(np.float32)
+    assert np.array_equal(orc.unpack_chunks([orc.pack_slices(x, S, B, axis)], B, axis), x)
+    cshape = (24, L // S) if axis == 1 else (L // S, 24)
+    peers = [[rng.standard_normal(cshape).astype(np.float32) for _ in range(S)] for _ in range(parts)]
+    for w in range(parts):
+        got = orc.unpack_chunks(peers, B, axis, window=w, parts=parts)
+        want = orc.assemble_ls(peers, 1, parts, w, S, B) if axis == 1 else orc.assemble_rs(peers, parts, 1, w, S, B)
+        assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
+        if parts <= 2:  # a two-term fp32 sum has one rounding whatever the order
+            assert np.array_equal(got, want)
+        got16 = orc.unpack_chunks(peers, B, axis, window=w, parts=parts, out_dtype="bf16")
+        assert np.array_equal(got16, orc.bf16_round(got))
+
+
 # ---------------------------------------------------------------- bf16 rounding
 def test_bf16_round_matches_torch_and_special_values():
     rng = np.random.default_rng(1)
