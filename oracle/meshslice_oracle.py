@@ -19,6 +19,8 @@ The tests pin one against the other, both against exact rational arithmetic on t
 reference's own ``arange`` fixtures (MeshFlowCPU.ipynb cells 2-4, TensorParallel.py:425-457),
 and against the C restatement in ``ms_oracle.c``.
 
+``pack_slices`` / ``unpack_chunks`` restate the layout statements either side of the contraction on their own.
+
 Parity status of every function: pinned (see tests/test_oracle_*.py).  What is NOT pinned,
 because only an import of JAX could pin it and JAX is not installed: the bit-exact rounding
 order of XLA:CPU's dot_general and the sample stream of ``jax.random.normal`` used by
