@@ -195,6 +195,12 @@ def main():
         extra["os_s4_fused_gelu_ms"] = round(_events(lambda: ms.gemm_os(A, B, out=C, activation="gelu"), 10), 4)
         extra["os_s4_then_separate_gelu_ms"] = round(_events(
             lambda: torch.nn.functional.gelu(ms.gemm_os(A, B, out=C), approximate="tanh"), 10), 4)
+        # what this device sustains on the bare MFMA instruction stream (no memory traffic) for operands drawn
+        # like X: the practical, power-limited ceiling beside the data-sheet peak
+        from meshslice_amd.local_gemm import mfma_stream_rate
+        stream_tf = mfma_stream_rate(X[:8, :512].contiguous().reshape(-1)) / 1e12
+        extra["mfma_stream_ceiling_tflops"] = round(stream_tf, 1)
+        extra["achieved_over_mfma_stream_ceiling"] = round(value / stream_tf, 4)
 
     out = {
         "metric": "per-device sliced GEMM throughput (GPT-3 FFN up-proj, output-stationary, S=4)",

@@ -156,6 +156,18 @@ int ms_unpack_chunks(const void *const *chunks, int P, int S, int ld_chunk, int 
                      int rows, int cols, int axis, int B, void *out, int ld_out,
                      int in_dtype, int out_dtype, void *stream);
 
+/* Measurement aid (no counterpart in the reference): the rate at which the current device sustains a bare
+ * stream of v_mfma_f32_32x32x16_bf16, the instruction the bf16 kernels are built on — one wave per SIMD,
+ * operands and accumulators resident in registers, no memory traffic.  Under its package power limit the
+ * device clocks this stream below the data-sheet frequency, by an amount that depends on the operand
+ * data, so this is the practical ceiling against which a kernel's achieved rate can be read.
+ * operands: 8 fragments x 64 lanes x 8 bf16 (8 KB, 16-byte aligned), typically the same distribution as
+ * the GEMM's inputs; sink: one float per launched thread (256 x CU count floats) that receives the sums;
+ * iters: loop trips of 64 MFMAs per wave.  Launches warmup + reps kernels on `stream`, waits, and
+ * returns the mean milliseconds per launch in *ms_out and the FLOPs of one launch in *flops_per_launch. */
+int ms_probe_mfma_stream(const void *operands, float *sink, int iters, int warmup, int reps,
+                         float *ms_out, double *flops_per_launch, void *stream);
+
 /* Tuning knob for experiments: selects the bf16 kernel variant used by later calls on this
  * thread (0 = library default).  Unknown ids are rejected with MS_ERR_ARG. */
 int ms_set_variant(int variant);

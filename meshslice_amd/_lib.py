@@ -31,7 +31,7 @@ EXPORTS = (
     "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
     "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex",
     "ms_time_os", "ms_time_ls", "ms_time_rs",
-    "ms_pack_slices", "ms_unpack_chunks",
+    "ms_pack_slices", "ms_unpack_chunks", "ms_probe_mfma_stream",
 )
 
 _lock = threading.Lock()
@@ -73,6 +73,9 @@ def _declare(lib):
     # chunks, P, S, ld_chunk, row_off, col_off, rows, cols, axis, B, out, ld_out, in_dtype, out_dtype, stream
     lib.ms_unpack_chunks.argtypes = [vpp, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_vp, c_int, c_int, c_int, c_vp]
     lib.ms_unpack_chunks.restype = c_int
+    # operands, sink, iters, warmup, reps, ms_out, flops_per_launch, stream
+    lib.ms_probe_mfma_stream.argtypes = [c_vp, c_vp, c_int, c_int, c_int, fp, ctypes.POINTER(ctypes.c_double), c_vp]
+    lib.ms_probe_mfma_stream.restype = c_int
     for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_time_os", "ms_time_ls", "ms_time_rs"):
         getattr(lib, n).restype = c_int
 

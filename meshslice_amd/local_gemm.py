@@ -185,3 +185,27 @@ def time_call(flow: str, operands, out, warmup: int = 5, reps: int = 20) -> List
         raise ValueError(f"unknown dataflow {flow!r}")
     _lib.check(rc)
     return list(ms)
+
+
+def mfma_stream_rate(operands: Optional[torch.Tensor] = None, iters: int = 4000, warmup: int = 20, reps: int = 200) -> float:
+    """FLOP/s that the current GPU sustains on a bare stream of the bf16 MFMA instruction the kernels are
+    built on (``ms_probe_mfma_stream``): the practical ceiling, under the device's power limit, for the
+    operand data given (default: N(0,1) values rounded to bf16, seed 0).  ``warmup + reps`` launches of about
+    a millisecond each, so the figure is the sustained one."""
+    dev = torch.device("cuda", torch.cuda.current_device())
+    if operands is None:
+        g = torch.Generator(device="cpu").manual_seed(0)
+        operands = torch.randn(8 * 64 * 8, generator=g).to(torch.bfloat16).to(dev)
+    if not (operands.is_cuda and operands.dtype == torch.bfloat16 and operands.is_contiguous() and operands.numel() >= 8 * 64 * 8):
+        raise ValueError("operands must be a contiguous bf16 GPU tensor of at least 4096 elements")
+    with torch.cuda.device(operands.device):
+        cus = _lib.load().ms_query(_lib.MS_QUERY_CU_COUNT)
+    if cus <= 0:
+        raise _lib.MeshSliceError("could not read the compute-unit count of the device")
+    sink = torch.empty(256 * int(cus), dtype=torch.float32, device=operands.device)
+    ms, fl = ctypes.c_float(0.0), ctypes.c_double(0.0)
+    with torch.cuda.device(operands.device):
+        rc = _lib.load().ms_probe_mfma_stream(ctypes.c_void_p(operands.data_ptr()), ctypes.c_void_p(sink.data_ptr()),
+                                              int(iters), int(warmup), int(reps), ctypes.byref(ms), ctypes.byref(fl), _stream())
+    _lib.check(rc)
+    return fl.value / (ms.value * 1e-3)

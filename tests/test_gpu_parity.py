@@ -460,3 +460,18 @@ def test_fused_epilogue_rejections():
         ms.gemm_os([h], [h], residual=torch.zeros((64, 32), dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(ValueError):
         ms.gemm_os([h], [h], row_moments=(torch.zeros(63, device="cuda"), None))
+
+
+def test_mfma_stream_probe_reports_a_plausible_rate():
+    """The measurement aid runs, stays under the data-sheet peak and above a tenth of it, and rejects bad arguments."""
+    from meshslice_amd.local_gemm import mfma_stream_rate
+    rate = mfma_stream_rate(iters=500, warmup=2, reps=5)
+    assert 0.25e15 < rate < 2.5166e15 * 1.02
+    L = _lib.load()
+    ms_out, fl = ctypes.c_float(), ctypes.c_double()
+    x = torch.zeros(4096, dtype=torch.bfloat16, device="cuda"); sink = torch.zeros(256 * 256, device="cuda")
+    assert L.ms_probe_mfma_stream(None, ctypes.c_void_p(sink.data_ptr()), 10, 0, 1, ctypes.byref(ms_out), ctypes.byref(fl), None) == _lib.MS_ERR_ARG
+    assert L.ms_probe_mfma_stream(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(sink.data_ptr()), 0, 0, 1, ctypes.byref(ms_out), ctypes.byref(fl), None) == _lib.MS_ERR_ARG
+    with pytest.raises(ValueError):
+        mfma_stream_rate(torch.zeros(16, dtype=torch.bfloat16, device="cuda"))
+
