@@ -16,7 +16,8 @@ by having one GPU and no tracing compiler:
   the running sum in the input dtype, :167);
 * the sliced OS body rejects ``K == 1``: the reference adds slice 0 twice in that case (:163,:172);
   use ``algorithm='collective'`` for the unsliced product;
-* the 'wang' and 'cannon' baselines are not built.
+* the ring baselines 'wang' and 'cannon' (:34-149, :218-342) drive the same kernels with 2 * size
+  half-block slices in ring order; the hops themselves are host index arithmetic.
 """
 from __future__ import annotations
 
@@ -139,6 +140,104 @@ def MeshFlow_RS(X, W, i, j, R, C, K, B):
 
 
 # ------------------------------------------------------------------------------------------------
+# ring baselines.  In the reference the halves of one operand (or of the partial output) travel round a
+# mesh axis with ppermute, one hop per step, and each step multiplies two half-blocks (Wang_OS/LS/RS,
+# reference :34-149; Cannon_OS/LS/RS, :218-342).  Seen from one device that is the same local
+# contraction as the unsliced body, cut into 2 * size half-blocks taken in the order of their arrival:
+# one kernel call with 2 * size slices (OS) or 2 * size chunks written to their places in the device's
+# partial output (LS / RS).  The reference reads the device's ring position with ``jax.lax.ax_index``,
+# a name JAX does not have; the position is taken here as ``axis_index`` gives it.
+# ------------------------------------------------------------------------------------------------
+
+def _ring_order(algorithm: str, dataflow: str, R: int, C: int, i: int, j: int):
+    """[(block, half)] in step order for device (i, j).  Wang: ring = the mesh row; the low halves come from
+    the left (block j, j-1, ..), the high halves from the right (j, j+1, ..); for LS the partial outputs
+    travel instead and a device works on block j-1-t / j+1+t in step t (reference :45-59, :76-89,
+    :132-146).  Cannon (square mesh): both start at k = (i + j) % N, low halves move on to k+1, k+2, ..,
+    high halves to k-1, k-2, .. (:235-259, :268-294, :309-335)."""
+    if algorithm == "wang":
+        if dataflow == "ls":
+            return [p for t in range(C) for p in (((j - 1 - t) % C, 0), ((j + 1 + t) % C, 1))]
+        return [p for t in range(C) for p in (((j - t) % C, 0), ((j + t) % C, 1))]
+    k = (i + j) % C
+    return [p for t in range(C) for p in (((k + t) % C, 0), ((k - t) % C, 1))]
+
+
+def _usable(views: Sequence[torch.Tensor]) -> List[torch.Tensor]:
+    """The views themselves if the kernels can address all of them in place, else contiguous copies of all
+    (slices of one call share a leading dimension)."""
+    if all(_own(v) is v for v in views):
+        return list(views)
+    return [v.contiguous() for v in views]
+
+
+def _ring_os(algorithm, X, W, i, j, R, C):
+    Wj = _gather([W[ii][j] for ii in range(R)], 0)                       # [Kd, n/C]
+    _need(X[i][j].shape[1], 2, "columns of an X shard"); _need(Wj.shape[0], 2 * C, "gathered rows of W")
+    h = Wj.shape[0] // C // 2
+    order = _ring_order(algorithm, "os", R, C, i, j)
+    A = _usable([X[i][b][:, hi * h:(hi + 1) * h] for b, hi in order])
+    Bs = [Wj[(2 * b + hi) * h:(2 * b + hi + 1) * h] for b, hi in order]
+    return local_gemm.gemm_os(A, Bs)
+
+
+def _ring_ls(algorithm, X, W, i, j, R, C):
+    Wj = _gather([W[ii][j] for ii in range(R)], 0)                       # [O, I/C]
+    _need(Wj.shape[0], 2 * C, "gathered rows of W")
+    h = Wj.shape[0] // C // 2
+    order = _ring_order(algorithm, "ls", R, C, i, j)
+    Xij = _own(X[i][j])
+    part = torch.empty((Xij.shape[0], Wj.shape[0]), dtype=torch.float32, device=Xij.device)
+    outs = [part[:, (2 * b + hi) * h:(2 * b + hi + 1) * h] for b, hi in order]
+    if any(o.data_ptr() % 16 for o in outs):
+        raise ValueError(f"half-blocks of {h} output columns are not 16-byte aligned")
+    local_gemm.gemm_ls(Xij, [Wj[(2 * b + hi) * h:(2 * b + hi + 1) * h] for b, hi in order], out=outs)
+    return [part]
+
+
+def _ring_rs(algorithm, X, W, i, j, R, C):
+    _need(X[i][j].shape[1], 2, "columns of an X shard")
+    h = X[i][j].shape[1] // 2
+    order = _ring_order(algorithm, "rs", R, C, i, j)
+    Xs = _usable([X[i][b][:, hi * h:(hi + 1) * h] for b, hi in order])
+    Wij = _own(W[i][j])
+    part = torch.empty((2 * h * C, Wij.shape[1]), dtype=torch.float32, device=Wij.device)
+    local_gemm.gemm_rs(Xs, Wij, out=[part[(2 * b + hi) * h:(2 * b + hi + 1) * h] for b, hi in order])
+    return [part]
+
+
+def Wang_OS(X, W, i, j, R, C, K, B):
+    """reference :34-61."""
+    return _ring_os("wang", X, W, i, j, R, C)
+
+
+def Wang_LS(X, W, i, j, R, C, K, B):
+    """reference :64-90; returns the device's whole partial output ``X_ij @ Wj^T`` (what the travelling
+    half-blocks sum up over the mesh row)."""
+    return _ring_ls("wang", X, W, i, j, R, C)
+
+
+def Wang_RS(X, W, i, j, R, C, K, B):
+    """reference :92-149 (the branch it takes, :120-149); returns the device's partial ``Xi^T @ W_ij``."""
+    return _ring_rs("wang", X, W, i, j, R, C)
+
+
+def Cannon_OS(X, W, i, j, R, C, K, B):
+    """reference :218-260."""
+    return _ring_os("cannon", X, W, i, j, R, C)
+
+
+def Cannon_LS(X, W, i, j, R, C, K, B):
+    """reference :262-300."""
+    return _ring_ls("cannon", X, W, i, j, R, C)
+
+
+def Cannon_RS(X, W, i, j, R, C, K, B):
+    """reference :302-342."""
+    return _ring_rs("cannon", X, W, i, j, R, C)
+
+
+# ------------------------------------------------------------------------------------------------
 # mesh completion: what psum_scatter + the (.., K, B) interleave do with the partial chunks
 # ------------------------------------------------------------------------------------------------
 
@@ -251,10 +350,13 @@ class SPMD:
         if algorithm == "collective":
             self.funcs = {"os": Collective_OS, "ls": Collective_LS, "rs": Collective_RS}
             self.sliced = False
-        elif algorithm in ("wang", "cannon"):
-            raise NotImplementedError(
-                f"algorithm {algorithm!r} (a comparison baseline of the reference) is not part of this build; "
-                "use 'collective' or 'meshflow'")
+        elif algorithm == "wang":
+            self.funcs = {"os": Wang_OS, "ls": Wang_LS, "rs": Wang_RS}
+            self.sliced = False
+        elif algorithm == "cannon":
+            assert mesh.devices.shape[0] == mesh.devices.shape[1], "cannon needs a square mesh"
+            self.funcs = {"os": Cannon_OS, "ls": Cannon_LS, "rs": Cannon_RS}
+            self.sliced = False
         else:  # like the reference, any other name selects the sliced MeshFlow bodies
             self.funcs = {"os": MeshFlow_OS, "ls": MeshFlow_LS, "rs": MeshFlow_RS}
             self.sliced = True

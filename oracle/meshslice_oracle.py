@@ -427,6 +427,191 @@ def literal_meshflow(dataflow, X, W, R, C, K, B):
     return {"os": literal_meshflow_os, "ls": literal_meshflow_ls, "rs": literal_meshflow_rs}[dataflow](X, W, R, C, K, B)
 
 
+# --------------------------------------------------------------------------------------
+# literal whole-mesh emulation of the ring baselines (Wang, Cannon)
+# --------------------------------------------------------------------------------------
+# The reference's bodies read the device's position with ``jax.lax.ax_index`` (TensorParallel.py:37,67,
+# 122,219-220,264-265,305-306), a name JAX does not have; they are restated here with the position taken
+# as ``axis_index`` would give it, which is the only reading under which they compute the product.
+
+def _ppermute(blocks, R, C, over, shift):
+    """jax.lax.ppermute with perm [(p, (p + shift) % size)]: every device sends its block to the peer
+    ``shift`` places further along mesh axis ``over``; returned is what each device receives."""
+    out = [[None] * C for _ in range(R)]
+    for i in range(R):
+        for j in range(C):
+            if over == "col":
+                out[i][(j + shift) % C] = blocks[i][j]
+            else:
+                out[(i + shift) % R][j] = blocks[i][j]
+    return out
+
+
+def _grid(f, R, C):
+    return [[f(i, j) for j in range(C)] for i in range(R)]
+
+
+def literal_wang_os(X, W, R, C):
+    """Wang_OS (TensorParallel.py:34-61): W gathered over the rows; the two halves of the X shard travel
+    round the mesh row in opposite directions, each multiplied with the matching half-block of W."""
+    Xs, Ws = _shards(X, R, C), _shards(W, R, C)
+    Wj = _all_gather(Ws, R, C, "row", 0)
+    size = C
+    up = lambda b: _ppermute(b, R, C, "col", +1)
+    dn = lambda b: _ppermute(b, R, C, "col", -1)
+    B = Wj[0][0].shape[0] // size // 2
+    wb = lambda i, j, blk, hi: _dyn_slice(Wj[i][j], (2 * blk + hi) * B, B, 0)
+    lo = _grid(lambda i, j: np.split(Xs[i][j], 2, axis=1)[0], R, C)
+    hi = _grid(lambda i, j: np.split(Xs[i][j], 2, axis=1)[1], R, C)
+    out = _grid(lambda i, j: lo[i][j] @ wb(i, j, j, 0) + hi[i][j] @ wb(i, j, j, 1), R, C)
+    lo, hi = up(lo), dn(hi)
+    for ii in range(1, size):
+        lo2, hi2 = up(lo), dn(hi)
+        out = _grid(lambda i, j: out[i][j] + lo[i][j] @ wb(i, j, (j - ii) % size, 0) + hi[i][j] @ wb(i, j, (j + ii) % size, 1), R, C)
+        lo, hi = lo2, hi2
+    return _unshard(out)
+
+
+def literal_wang_ls(X, W, R, C):
+    """Wang_LS (TensorParallel.py:64-90): W ([out, in]) gathered over the rows; partial outputs for one
+    half-block of the output columns at a time travel round the mesh row and pick up every device's term."""
+    Xs, Ws = _shards(X, R, C), _shards(W, R, C)
+    Wj = _all_gather(Ws, R, C, "row", 0)
+    size = C
+    up = lambda b: _ppermute(b, R, C, "col", +1)
+    dn = lambda b: _ppermute(b, R, C, "col", -1)
+    B = Wj[0][0].shape[0] // size // 2
+    wb = lambda i, j, blk, hi: _dyn_slice(Wj[i][j], (2 * blk + hi) * B, B, 0)
+    dot = lambda a, b: np.einsum("bi,oi->bo", a, b)
+    ylo = _grid(lambda i, j: dot(Xs[i][j], wb(i, j, (j - 1) % size, 0)), R, C)
+    yhi = _grid(lambda i, j: dot(Xs[i][j], wb(i, j, (j + 1) % size, 1)), R, C)
+    for ii in range(1, size):
+        ylo, yhi = up(ylo), dn(yhi)
+        ylo = _grid(lambda i, j: ylo[i][j] + dot(Xs[i][j], wb(i, j, (j - ii - 1) % size, 0)), R, C)
+        yhi = _grid(lambda i, j: yhi[i][j] + dot(Xs[i][j], wb(i, j, (j + ii + 1) % size, 1)), R, C)
+    return _unshard(_grid(lambda i, j: np.concatenate([ylo[i][j], yhi[i][j]], axis=1), R, C))
+
+
+def literal_wang_rs(X, W, R, C):
+    """Wang_RS, the branch the reference takes (TensorParallel.py:120-149): the halves of the X shard
+    ([in, tokens]) travel round the mesh row; every device fills its [tokens, out/C] partial block by block,
+    then psum_scatter over the rows."""
+    Xs, Ws = _shards(X, R, C), _shards(W, R, C)
+    size = C
+    up = lambda b: _ppermute(b, R, C, "col", +1)
+    dn = lambda b: _ppermute(b, R, C, "col", -1)
+    dot = lambda a, b: np.einsum("ib,io->bo", a, b)
+    Yj = _grid(lambda i, j: np.zeros((Xs[i][j].shape[1] * C, Ws[i][j].shape[1]), X.dtype), R, C)
+    B = Yj[0][0].shape[0] // size // 2
+
+    def put(y, blk, start):
+        y = y.copy(); y[start:start + blk.shape[0]] = blk
+        return y
+    Yj = _grid(lambda i, j: put(Yj[i][j], dot(Xs[i][j], Ws[i][j]), 2 * (j % size) * B), R, C)
+    lo = up(_grid(lambda i, j: np.split(Xs[i][j], 2, axis=1)[0], R, C))
+    hi = dn(_grid(lambda i, j: np.split(Xs[i][j], 2, axis=1)[1], R, C))
+    for ii in range(1, size):
+        Yj = _grid(lambda i, j: put(Yj[i][j], dot(lo[i][j], Ws[i][j]), 2 * ((j - ii) % size) * B), R, C)
+        Yj = _grid(lambda i, j: put(Yj[i][j], dot(hi[i][j], Ws[i][j]), 2 * ((j + ii) % size) * B + B), R, C)
+        lo, hi = up(lo), dn(hi)
+    return _unshard(_psum_scatter(Yj, R, C, "row", 0))
+
+
+def literal_cannon_os(X, W, R, C):
+    """Cannon_OS (TensorParallel.py:218-260), square mesh: device (r, c) starts at half-block pair
+    k = (c + r) % N; the halves of both operands move on in opposite directions every step."""
+    assert R == C
+    N = C
+    Xs, Ws = _shards(X, R, C), _shards(W, R, C)
+    Xi = _all_gather(Xs, R, C, "col", 1)
+    Wj = _all_gather(Ws, R, C, "row", 0)
+    B = Xi[0][0].shape[1] // N // 2
+    k = lambda i, j: (j + i) % N
+    xl = _grid(lambda i, j: _dyn_slice(Xi[i][j], 2 * k(i, j) * B, B, 1), R, C)
+    xh = _grid(lambda i, j: _dyn_slice(Xi[i][j], (2 * k(i, j) + 1) * B, B, 1), R, C)
+    wl = _grid(lambda i, j: _dyn_slice(Wj[i][j], 2 * k(i, j) * B, B, 0), R, C)
+    wh = _grid(lambda i, j: _dyn_slice(Wj[i][j], (2 * k(i, j) + 1) * B, B, 0), R, C)
+    out = _grid(lambda i, j: xl[i][j] @ wl[i][j] + xh[i][j] @ wh[i][j], R, C)
+    step = lambda xl, xh, wl, wh: (_ppermute(xl, R, C, "col", -1), _ppermute(xh, R, C, "col", +1),
+                                   _ppermute(wl, R, C, "row", -1), _ppermute(wh, R, C, "row", +1))
+    xl, xh, wl, wh = step(xl, xh, wl, wh)
+    for _ in range(1, N):
+        nxt = step(xl, xh, wl, wh)
+        out = _grid(lambda i, j: out[i][j] + xl[i][j] @ wl[i][j] + xh[i][j] @ wh[i][j], R, C)
+        xl, xh, wl, wh = nxt
+    return _unshard(out)
+
+
+def literal_cannon_ls(X, W, R, C):
+    """Cannon_LS (TensorParallel.py:262-300)."""
+    assert R == C
+    N = C
+    Xs, Ws = _shards(X, R, C), _shards(W, R, C)
+    k = lambda i, j: (j + i) % N
+    B = Ws[0][0].shape[0] // 2
+    Wj = _all_gather(Ws, R, C, "row", 0)
+    wl = _grid(lambda i, j: _dyn_slice(Wj[i][j], 2 * k(i, j) * B, B, 0), R, C)
+    wh = _grid(lambda i, j: _dyn_slice(Wj[i][j], (2 * k(i, j) + 1) * B, B, 0), R, C)
+    dot = lambda a, b: np.einsum("bi,oi->bo", a, b)
+    yl = _map2(dot, Xs, wl, R, C)
+    yh = _map2(dot, Xs, wh, R, C)
+    for _ in range(1, N):
+        wl, wh = _ppermute(wl, R, C, "row", -1), _ppermute(wh, R, C, "row", +1)
+        yl, yh = _ppermute(yl, R, C, "col", -1), _ppermute(yh, R, C, "col", +1)
+        yl = _map2(lambda y, p: y + p, yl, _map2(dot, Xs, wl, R, C), R, C)
+        yh = _map2(lambda y, p: y + p, yh, _map2(dot, Xs, wh, R, C), R, C)
+    yl, yh = _ppermute(yl, R, C, "col", -1), _ppermute(yh, R, C, "col", +1)
+    Yik = _grid(lambda i, j: np.concatenate([yl[i][j], yh[i][j]], axis=1), R, C)
+    Yi = _all_gather(Yik, R, C, "col", 1)
+    return _unshard(_grid(lambda i, j: _dyn_slice(Yi[i][j], 2 * ((j - i) % N) * B, 2 * B, 1), R, C))
+
+
+def literal_cannon_rs(X, W, R, C):
+    """Cannon_RS (TensorParallel.py:302-342)."""
+    assert R == C
+    N = C
+    Xs, Ws = _shards(X, R, C), _shards(W, R, C)
+    k = lambda i, j: (j + i) % N
+    B = Xs[0][0].shape[1] // 2
+    Xi = _all_gather(Xs, R, C, "col", 1)
+    xl = _grid(lambda i, j: _dyn_slice(Xi[i][j], 2 * k(i, j) * B, B, 1), R, C)
+    xh = _grid(lambda i, j: _dyn_slice(Xi[i][j], (2 * k(i, j) + 1) * B, B, 1), R, C)
+    dot = lambda a, b: np.einsum("ib,io->bo", a, b)
+    yl = _map2(dot, xl, Ws, R, C)
+    yh = _map2(dot, xh, Ws, R, C)
+    for _ in range(1, N):
+        xl, xh = _ppermute(xl, R, C, "col", -1), _ppermute(xh, R, C, "col", +1)
+        yl, yh = _ppermute(yl, R, C, "row", -1), _ppermute(yh, R, C, "row", +1)
+        yl = _map2(lambda y, p: y + p, yl, _map2(dot, xl, Ws, R, C), R, C)
+        yh = _map2(lambda y, p: y + p, yh, _map2(dot, xh, Ws, R, C), R, C)
+    yl, yh = _ppermute(yl, R, C, "row", -1), _ppermute(yh, R, C, "row", +1)
+    Ykj = _grid(lambda i, j: np.concatenate([yl[i][j], yh[i][j]], axis=0), R, C)
+    Yj = _all_gather(Ykj, R, C, "row", 0)
+    return _unshard(_grid(lambda i, j: _dyn_slice(Yj[i][j], 2 * ((i - j) % N) * B, 2 * B, 0), R, C))
+
+
+def literal_ring(algorithm, dataflow, X, W, R, C):
+    return {("wang", "os"): literal_wang_os, ("wang", "ls"): literal_wang_ls, ("wang", "rs"): literal_wang_rs,
+            ("cannon", "os"): literal_cannon_os, ("cannon", "ls"): literal_cannon_ls,
+            ("cannon", "rs"): literal_cannon_rs}[(algorithm, dataflow)](X, W, R, C)
+
+
+# the order in which device (i, j) multiplies its 2 * size half-blocks (what its local kernel call is given)
+def ring_order(algorithm: str, dataflow: str, R: int, C: int, i: int, j: int):
+    """[(block, half)] in step order for device (i, j): block indexes the contraction (OS) or output (LS /
+    RS) range in units of two half-blocks.  Wang: the ring is the mesh row (size C), Cannon: N = R = C."""
+    if algorithm == "wang":
+        size = C
+        if dataflow == "os":
+            return [p for t in range(size) for p in (((j - t) % size, 0), ((j + t) % size, 1))]
+        if dataflow == "ls":
+            return [p for t in range(size) for p in (((j - 1 - t) % size, 0), ((j + 1 + t) % size, 1))]
+        return [p for t in range(size) for p in (((j - t) % size, 0), ((j + t) % size, 1))]
+    N = C
+    k = (i + j) % N
+    return [p for t in range(N) for p in (((k + t) % N, 0), ((k - t) % N, 1))]
+
+
 def dense(dataflow, X, W):
     """What each dataflow computes on the global operands (MeshFlowCPU.ipynb cells 2-3):
     OS ``X@W``; LS ``X@W^T``; RS ``X^T@W``."""

@@ -254,6 +254,41 @@ def test_meshflow_equals_collective_equals_dense(flow, R, C, K):
     assert orc.rel_frobenius(host(y_m), lit) <= TOL_BF16
 
 
+@pytest.mark.parametrize("algorithm,R,C", [("wang", 2, 4), ("wang", 4, 2), ("cannon", 2, 2), ("cannon", 4, 4)])
+@pytest.mark.parametrize("flow", ["os", "ls", "rs"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_ring_baselines_equal_dense_and_the_literal_emulation(flow, algorithm, R, C, dtype):
+    """SPMD(mesh, 'wang' | 'cannon'): every device multiplies its 2 * size half-blocks in ring order in one kernel
+    call; the whole-mesh result equals the dense product, the collective body's result and the literal emulation
+    of the reference's ring bodies; a device's partial equals the collective body's partial."""
+    rng = np.random.default_rng(R * 10 + C)
+    u = R * C * 2 * 8
+    shp = {"os": ((4 * R * 8, 2 * u), (2 * u, 3 * C * 8)), "ls": ((4 * R * 8, 2 * C * 16), (2 * u, 2 * C * 16)),
+           "rs": ((4 * R * 8, 2 * u), (4 * R * 8, 3 * C * 8))}[flow]
+    rnd = (lambda a: orc.bf16_round(a)) if dtype == torch.bfloat16 else (lambda a: a)
+    X = rnd(rng.standard_normal(shp[0]).astype(np.float32))
+    W = rnd(rng.standard_normal(shp[1]).astype(np.float32) * np.float32(0.1))
+    tol = TOL_BF16 if dtype == torch.bfloat16 else TOL_F32
+    mesh = Mesh(create_device_mesh((R, C)), ("row", "col"))
+    dX, dW = dev(X, dtype), dev(W, dtype)
+    ring = getattr(TP.SPMD(mesh, algorithm), flow.upper())()
+    coll = getattr(TP.SPMD(mesh, "collective"), flow.upper())()
+    y = ring(dX, dW)
+    want = orc.dense(flow, X, W)
+    assert y.dtype == dtype and tuple(y.shape) == want.shape
+    assert orc.rel_frobenius(host(y), want) <= tol
+    assert orc.rel_frobenius(host(y), orc.literal_ring(algorithm, flow, X.astype(np.float64), W.astype(np.float64), R, C)) <= tol
+    assert TP.allclose(y, coll(dX, dW))
+    i, j = R - 1, C // 2
+    got, ref = ring.device(i, j)(dX, dW), coll.device(i, j)(dX, dW)
+    if flow == "os":
+        blk = want[i * want.shape[0] // R:(i + 1) * want.shape[0] // R, j * want.shape[1] // C:(j + 1) * want.shape[1] // C]
+        assert orc.rel_frobenius(host(got), blk) <= tol
+    else:
+        assert len(got) == 1 and tuple(got[0].shape) == tuple(ref[0].shape)
+        assert orc.rel_frobenius(host(got[0]), host(ref[0])) <= 1e-6      # same terms per element, same k order
+
+
 @pytest.mark.parametrize("dataflow", ["os", "ls", "rs"])
 def test_sharded_ff_layer_forward_and_vjp(dataflow):
     """reference ShardedLayers.py:41-81: (fwd, dx, dw) = (OS,LS,RS) / (LS,OS,RS) / (RS,LS,OS)."""

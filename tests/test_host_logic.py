@@ -73,8 +73,11 @@ def test_spmd_surface_and_shape_errors():
     for name in ("systolic", "noff", "meshflow"):      # any other name selects the sliced bodies
         assert TP.SPMD(mesh, name).funcs["os"] is TP.MeshFlow_OS
     assert TP.SPMD(mesh, "collective").funcs["ls"] is TP.Collective_LS
-    with pytest.raises(NotImplementedError):
+    assert TP.SPMD(mesh, "wang").funcs["rs"] is TP.Wang_RS
+    with pytest.raises(AssertionError):                 # the reference asserts a square mesh (TensorParallel.py:359)
         TP.SPMD(mesh, "cannon")
+    sq = Mesh(create_device_mesh((2, 2)), ("row", "col"))
+    assert TP.SPMD(sq, "cannon").funcs["os"] is TP.Cannon_OS and not TP.SPMD(sq, "cannon").sliced
     f = s.OS()                                          # default K = 8
     assert f.K == 8
     with pytest.raises(ValueError):                     # 256/2 = 128 per shard, needs multiple of 8*8
@@ -85,6 +88,16 @@ def test_spmd_surface_and_shape_errors():
         f.device(4, 0)
     with pytest.raises(ValueError, match="K == 1"):
         TP.MeshFlow_OS(None, None, 0, 0, 4, 2, 1, 8)
+
+
+@pytest.mark.parametrize("algorithm,R,C", [("wang", 2, 4), ("wang", 4, 2), ("wang", 1, 3), ("cannon", 2, 2), ("cannon", 4, 4), ("cannon", 3, 3)])
+def test_ring_order_of_the_device_bodies_matches_the_oracle(algorithm, R, C):
+    for dataflow in ("os", "ls", "rs"):
+        for i in range(R):
+            for j in range(C):
+                order = TP._ring_order(algorithm, dataflow, R, C, i, j)
+                assert order == orc.ring_order(algorithm, dataflow, R, C, i, j)
+                assert sorted(order) == [(b, h) for b in range(C) for h in (0, 1)]      # every half-block exactly once
 
 
 # ---------------------------------------------------------------- cost model

@@ -87,6 +87,60 @@ def test_unpack_chunks_inverts_pack_and_matches_assembly(S, B, parts, axis):
         assert np.array_equal(got16, orc.bf16_round(got))
 
 
+# ---------------------------------------------------------------- ring baselines
+
+RING_MESHES = [("wang", 2, 4), ("wang", 4, 2), ("wang", 2, 2), ("wang", 1, 3), ("cannon", 2, 2), ("cannon", 4, 4), ("cannon", 3, 3)]
+
+
+@pytest.mark.parametrize("algorithm,R,C", RING_MESHES)
+@pytest.mark.parametrize("dataflow", ["os", "ls", "rs"])
+def test_literal_ring_baselines_equal_the_dense_product(algorithm, R, C, dataflow):
+    """Integer-valued operands: the statement-by-statement emulation of Wang_* / Cannon_* equals X@W, X@W^T,
+    X^T@W exactly (this is what fixes the reading of the device position and of every shift direction: any
+    other pairing of half-blocks misses or doubles a term)."""
+    rng = np.random.default_rng(R * 10 + C)
+    L = R * C * 2 * 3
+    shapes = {"os": ((L, L), (L, 2 * L)), "ls": ((L, L), (2 * L, L)), "rs": ((L, 2 * L), (L, L))}[dataflow]
+    X = rng.integers(-3, 4, shapes[0]).astype(np.float64)
+    W = rng.integers(-3, 4, shapes[1]).astype(np.float64)
+    assert np.array_equal(orc.literal_ring(algorithm, dataflow, X, W, R, C), orc.dense(dataflow, X, W))
+
+
+@pytest.mark.parametrize("algorithm,R,C", RING_MESHES)
+def test_ring_order_matches_labels_carried_round_the_ring(algorithm, R, C):
+    """ring_order() against labels moved with the same ppermute primitive and directions the literal
+    emulation uses: which (block, half) a device holds, or works on, at every step."""
+    lab = lambda h: [[(j, h) for j in range(C)] for _ in range(R)]
+    for dataflow in ("os", "ls", "rs"):
+        seen = [[[] for _ in range(C)] for _ in range(R)]
+        if algorithm == "wang":
+            lo, hi = lab(0), lab(1)
+            if dataflow == "ls":   # partial outputs travel: the device holding block b's partial adds its term
+                lo = [[((j - 1) % C, 0) for j in range(C)] for _ in range(R)]
+                hi = [[((j + 1) % C, 1) for j in range(C)] for _ in range(R)]
+            for t in range(C):
+                for i in range(R):
+                    for j in range(C):
+                        seen[i][j] += [lo[i][j], hi[i][j]]
+                if dataflow == "ls":   # the label a device receives is the block it must NOT redo: it works on the one before
+                    lo = [[((b - 1) % C, h) for b, h in row] for row in lo]
+                    hi = [[((b + 1) % C, h) for b, h in row] for row in hi]
+                else:
+                    lo, hi = orc._ppermute(lo, R, C, "col", +1), orc._ppermute(hi, R, C, "col", -1)
+        else:
+            lo = [[((i + j) % C, 0) for j in range(C)] for i in range(R)]
+            hi = [[((i + j) % C, 1) for j in range(C)] for i in range(R)]
+            for t in range(C):
+                for i in range(R):
+                    for j in range(C):
+                        seen[i][j] += [lo[i][j], hi[i][j]]
+                axis = "col" if dataflow != "ls" else "row"   # the operand halves that move: X along col (OS, RS), W along row (LS)
+                lo, hi = orc._ppermute(lo, R, C, axis, -1), orc._ppermute(hi, R, C, axis, +1)
+        for i in range(R):
+            for j in range(C):
+                assert seen[i][j] == orc.ring_order(algorithm, dataflow, R, C, i, j), (dataflow, i, j)
+
+
 # ---------------------------------------------------------------- bf16 rounding
 def test_bf16_round_matches_torch_and_special_values():
     rng = np.random.default_rng(1)
