@@ -194,6 +194,42 @@ def test_peer_major_gathered_slices_are_ingested_without_a_repack():
     assert orc.rel_frobenius(c_pm.cpu().numpy().astype(np.float64), c_rm.cpu().numpy().astype(np.float64)) <= 1e-6
 
 
+def test_device_step_is_capturable_in_a_hip_graph():
+    """One device's step of the LHS-stationary dataflow — cut the weight shard into slices, multiply, reduce and
+    interleave the chunks — captured once and replayed with new operand values each time; every replay equals
+    the eager result bit for bit (kernel launches only: no allocation, no memset inside the calls)."""
+    import meshslice_amd as ms
+    S, B = 4, 8
+    g = torch.Generator(device="cuda").manual_seed(31)
+    x = torch.randn((256, 512), generator=g, device="cuda").to(torch.bfloat16)
+    w = (torch.randn((768, 512), generator=g, device="cuda") * 0.05).to(torch.bfloat16)          # [out, in] shard
+    wsl = [torch.empty((768 // S, 512), dtype=torch.bfloat16, device="cuda") for _ in range(S)]
+    chunks = [torch.empty((256, 768 // S), dtype=torch.float32, device="cuda") for _ in range(S)]
+    y = torch.empty((256, 768), dtype=torch.bfloat16, device="cuda")
+
+    def step():
+        sl.pack_slices(w, S, B, 0, out=wsl)
+        ms.gemm_ls(x, wsl, out=chunks)
+        sl.unpack_chunks([chunks], B, 1, out=y)
+    step()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        x.copy_(torch.randn((256, 512), generator=g, device="cuda").to(torch.bfloat16))
+        w.mul_(-1.5)
+        step()
+        want = y.clone()
+        y.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want), f"replay {rep} differs from the eager step"
+        ref = x.double() @ w.double().t()
+        assert orc.rel_frobenius(y.double().cpu().numpy(), ref.cpu().numpy()) <= 1e-2
+
+
 def test_layout_calls_reject_bad_arguments():
     L = _lib.load()
     x = torch.zeros((64, 64), dtype=torch.bfloat16, device="cuda")
