@@ -195,6 +195,11 @@ def main():
         extra["os_s4_fused_gelu_ms"] = round(_events(lambda: ms.gemm_os(A, B, out=C, activation="gelu"), 10), 4)
         extra["os_s4_then_separate_gelu_ms"] = round(_events(
             lambda: torch.nn.functional.gelu(ms.gemm_os(A, B, out=C), approximate="tanh"), 10), 4)
+        # the layout kernels either side of the GEMM on the same [4096, 12288] bf16 shard: algorithmic GB/s (HBM roofline 8000)
+        from meshslice_amd.slice_layout import measure_rates
+        for label, t, nbytes in measure_rates(dtypes=(torch.bfloat16,), reduce_case=False, reps=24):
+            key = "layout_" + label.replace("bfloat16 ", "").replace(" of the shard", "").replace("=", "").replace(" ", "_").lower() + "_gbps"
+            extra[key] = round(nbytes / t / 1e9, 0)
         # what this device sustains on the bare MFMA instruction stream (no memory traffic) for operands drawn
         # like X: the practical, power-limited ceiling beside the data-sheet peak
         from meshslice_amd.local_gemm import mfma_stream_rate

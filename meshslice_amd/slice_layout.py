@@ -84,11 +84,12 @@ def unpack_chunks(chunks_by_peer: Sequence[Sequence[torch.Tensor]], B: int, axis
     return out
 
 
-def _rates(rows: int = 4096, cols: int = 12288, S: int = 8, B: int = 8, reps: int = 48, nset: int = 4) -> None:
-    """``python -m meshslice_amd.slice_layout``: time the layout kernels on [rows, cols] shards (HIP events on
-    the current stream) and print microseconds and algorithmic GB/s (bytes read once + bytes written once).
-    Launches rotate over ``nset`` separate source / destination sets, together larger than the 256 MB
-    last-level cache, so that every launch streams from and to HBM."""
+def measure_rates(rows: int = 4096, cols: int = 12288, S: int = 8, B: int = 8, reps: int = 48, nset: int = 4,
+                  dtypes=(torch.bfloat16, torch.float32), reduce_case: bool = True):
+    """Time the layout kernels on [rows, cols] shards (HIP events on the current stream).  Returns a list of
+    (label, seconds, algorithmic bytes): bytes read once + bytes written once.  Launches rotate over ``nset``
+    separate source / destination sets, together larger than the 256 MB last-level cache, so that every launch
+    streams from and to HBM."""
     def timed(f):
         for i in range(2 * nset):
             f(i % nset)
@@ -99,28 +100,29 @@ def _rates(rows: int = 4096, cols: int = 12288, S: int = 8, B: int = 8, reps: in
         e1.record(); torch.cuda.synchronize()
         return e0.elapsed_time(e1) / reps * 1e-3
 
-    for dtype in (torch.bfloat16, torch.float32):
+    out = []
+    for dtype in dtypes:
         name = str(dtype)[6:]
         xs = [torch.randn(rows, cols, device="cuda").to(dtype) for _ in range(nset)]
         ys = [torch.empty_like(x) for x in xs]
         nbytes = 2 * xs[0].numel() * xs[0].element_size()
-        t = timed(lambda i: ys[i].copy_(xs[i]))
-        print(f"{name:9s} device copy of the shard      {t * 1e6:7.1f} us {nbytes / t / 1e9:7.0f} GB/s", flush=True)
+        out.append((f"{name} device copy of the shard", timed(lambda i: ys[i].copy_(xs[i])), nbytes))
         for axis in (1, 0):
             slices = [pack_slices(x, S, B, axis) for x in xs]
-            t = timed(lambda i: pack_slices(xs[i], S, B, axis, out=slices[i]))
-            print(f"{name:9s} pack   axis {axis} S={S}            {t * 1e6:7.1f} us {nbytes / t / 1e9:7.0f} GB/s", flush=True)
-            t = timed(lambda i: unpack_chunks([slices[i]], B, axis, out=ys[i]))
-            print(f"{name:9s} unpack axis {axis} S={S} P=1        {t * 1e6:7.1f} us {nbytes / t / 1e9:7.0f} GB/s", flush=True)
+            out.append((f"{name} pack axis {axis} S={S}", timed(lambda i: pack_slices(xs[i], S, B, axis, out=slices[i])), nbytes))
+            out.append((f"{name} unpack axis {axis} S={S} P=1", timed(lambda i: unpack_chunks([slices[i]], B, axis, out=ys[i])), nbytes))
         del xs, ys, slices
-    # what follows the LHS-stationary GEMM of the large configuration on a 4-wide mesh row: 4 peers' 8 fp32
-    # chunks [rows, cols / 8], this device keeps a quarter of each, bf16 shard out
-    peers = [[[torch.randn(rows, cols // S, device="cuda") for _ in range(S)] for _ in range(4)] for _ in range(2)]
-    out = torch.empty(rows, cols // 4, dtype=torch.bfloat16, device="cuda")
-    nbytes = 4 * S * rows * (cols // S // 4) * 4 + out.numel() * 2
-    t = timed(lambda i: unpack_chunks(peers[i % 2], B, 1, window=1, parts=4, out=out))
-    print(f"fp32->bf16 reduce 4 peers + unpack axis 1 S={S} {t * 1e6:7.1f} us {nbytes / t / 1e9:7.0f} GB/s", flush=True)
+    if reduce_case:
+        # what follows the LHS-stationary GEMM of the large configuration on a 4-wide mesh row: 4 peers' S fp32
+        # chunks [rows, cols / S], this device keeps a quarter of each, bf16 shard out
+        peers = [[[torch.randn(rows, cols // S, device="cuda") for _ in range(S)] for _ in range(4)] for _ in range(2)]
+        y = torch.empty(rows, cols // 4, dtype=torch.bfloat16, device="cuda")
+        nbytes = 4 * S * rows * (cols // S // 4) * 4 + y.numel() * 2
+        out.append((f"fp32->bf16 reduce 4 peers + unpack axis 1 S={S}", timed(lambda i: unpack_chunks(peers[i % 2], B, 1, window=1, parts=4, out=y)), nbytes))
+    return out
 
 
 if __name__ == "__main__":
-    _rates()
+    # python -m meshslice_amd.slice_layout: microseconds and algorithmic GB/s of every layout kernel
+    for label, t, nbytes in measure_rates():
+        print(f"{label:48s} {t * 1e6:7.1f} us {nbytes / t / 1e9:7.0f} GB/s", flush=True)
