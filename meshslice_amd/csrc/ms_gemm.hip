@@ -33,14 +33,18 @@ MS_INSTANTIATE_RING(256, 256, 64, 2, 2, 4)
 MS_INSTANTIATE_RING(256, 192, 64, 2, 2, 2)
 MS_INSTANTIATE_RING(192, 256, 64, 2, 2, 2)
 #undef MS_INSTANTIATE_RING
-template __global__ void msk::gemm_bf16_big_kernel<true, false, true, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_big_kernel<true, false, false, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_big_kernel<true, false, true, true>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_big_kernel<true, false, false, true>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_big_kernel<true, true, false, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_big_kernel<true, true, true, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_big_kernel<false, false, false, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_big_kernel<false, false, true, false>(const msk::GemmArgs);
+#define MS_INSTANTIATE_BIG(TM, TN)                                                                             \
+  template __global__ void msk::gemm_bf16_big_kernel<TM, TN, true, false, true, false>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_big_kernel<TM, TN, true, false, false, false>(const msk::GemmArgs);  \
+  template __global__ void msk::gemm_bf16_big_kernel<TM, TN, true, false, true, true>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_bf16_big_kernel<TM, TN, true, false, false, true>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_big_kernel<TM, TN, true, true, false, false>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_big_kernel<TM, TN, true, true, true, false>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_bf16_big_kernel<TM, TN, false, false, false, false>(const msk::GemmArgs); \
+  template __global__ void msk::gemm_bf16_big_kernel<TM, TN, false, false, true, false>(const msk::GemmArgs);
+MS_INSTANTIATE_BIG(4, 6)
+MS_INSTANTIATE_BIG(6, 3)
+#undef MS_INSTANTIATE_BIG
 
 namespace {
 thread_local char g_err[512] = "";
@@ -149,8 +153,8 @@ void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
   if constexpr (!BIG) {
     msk::gemm_bf16_ring_kernel<BM, BN, BK_, NS, WGM, WGN, AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
   } else {
-    static_assert(BM == 256 && BN == 384 && BK_ == 64 && NS == 2 && WGM == 2 && WGN == 2, "the big-tile kernel has one shape");
-    msk::gemm_bf16_big_kernel<AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && BK_ == 64 && NS == 2 && WGM == 2 && WGN == 2, "the big-tile kernels are 2 x 2 waves on two 64-deep stages");
+    msk::gemm_bf16_big_kernel<BM / 64, BN / 64, AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
   }
 }
 
@@ -202,11 +206,12 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
 //   1: 256x256, 4 waves, 2 x 64     2: 256x256, 8 waves, 4 x 32     3: 128x128, 4 waves, 2 x 64
 //   4: 256x256, 4 waves, 4 x 32     5: 256x192, 4 waves, 4 x 32     6: 192x256, 4 waves, 4 x 32
 //   7: 256x256, 8 waves, 2 x 64     8: 256x192, 4 waves, 2 x 64     9: 192x256, 4 waves, 2 x 64
-//  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel)
+//  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel<4, 6>)     11: 384x192, 4 waves, 2 x 64 (gemm_bf16_big_kernel<6, 3>)
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
 // ceil(tiles / CUs) rounds of one tile per CU, so the estimate is rounds x tile area / relative tile
-// efficiency (measured on the GPT-3-sized product, per flop, 256x256 = 1: the 256x384 tile reaches 1.06
-// with a k-contiguous A and 0.8 without, 192-wide tiles about 0.93, 128x128 tiles about 0.55).  The
+// efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile reaches 1.06
+// with a k-contiguous A and 1.02 without, the 384x192 tile 1.04 and 1.0, 192-wide ring tiles about 0.93,
+// 128x128 tiles about 0.55).  The
 // ring-kernel defaults use four waves over two 64-deep stages when an operand is k-contiguous: whole
 // 128-byte lines per request, half as many barriers as 32-deep stages.
 int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
@@ -214,10 +219,11 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   int v = g_variant;
   if (v == 0) {
     struct Cand { int v, bm, bn; double eff; };
-    // with two m/n-contiguous operands (RS) the 32-deep four-stage ring measures 3 % faster than the 64-deep one
+    // with two m/n-contiguous operands (RS) the 32-deep four-stage ring measures 3 % faster than the 64-deep one,
+    // and the hand-scheduled tiles gain less over the 256x256 ring than with a k-contiguous operand
     const bool rs = p.flow == RS;
-    const Cand cands[] = {{rs ? 4 : 1, 256, 256, 1.0}, {10, 256, 384, rs ? 0.80 : 1.06}, {rs ? 5 : 8, 256, 192, 0.93},
-                          {rs ? 6 : 9, 192, 256, 0.93}, {3, 128, 128, 0.55}};
+    const Cand cands[] = {{rs ? 4 : 1, 256, 256, 1.0},           {10, 256, 384, rs ? 1.02 : 1.06}, {11, 384, 192, rs ? 1.0 : 1.04},
+                          {rs ? 5 : 8, 256, 192, rs ? 0.95 : 0.93}, {rs ? 6 : 9, 192, 256, rs ? 0.95 : 0.93}, {3, 128, 128, 0.55}};
     const long chunks = p.flow == OS ? 1 : p.S;
     double best = 0;
     for (const Cand &c : cands) {
@@ -238,6 +244,7 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
     case 8: return launch_bf16_tile<256, 192, 2, 2, 64, 2>(p, dev, stream);
     case 9: return launch_bf16_tile<192, 256, 2, 2, 64, 2>(p, dev, stream);
     case 10: return launch_bf16_tile<256, 384, 2, 2, 64, 2, true>(p, dev, stream);
+    case 11: return launch_bf16_tile<384, 192, 2, 2, 64, 2, true>(p, dev, stream);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }
@@ -344,7 +351,7 @@ MS_API long ms_query(int what) {
 }
 
 MS_API int ms_set_variant(int variant) {
-  if (variant < 0 || variant > 10) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  if (variant < 0 || variant > 11) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
   g_variant = variant;
   return MS_OK;
 }
