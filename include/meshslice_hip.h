@@ -43,6 +43,8 @@ extern "C" {
 #define MS_QUERY_IS_GFX950 2    /* 1 if the current device is gfx950 */
 #define MS_QUERY_LDS_BYTES 3    /* LDS bytes per workgroup */
 #define MS_QUERY_MAX_SLICES 4   /* MS_MAX_SLICES */
+#define MS_QUERY_LAST_LAUNCHES 5 /* kernels launched by the calling thread's last ms_gemm_* call (a product whose tiles
+                                   would leave much of the last round of compute units idle is done in two launches) */
 
 /* Library version, major*10000 + minor*100 + patch. */
 int ms_version(void);

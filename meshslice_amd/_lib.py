@@ -21,6 +21,7 @@ MS_QUERY_CLOCK_KHZ = 1
 MS_QUERY_IS_GFX950 = 2
 MS_QUERY_LDS_BYTES = 3
 MS_QUERY_MAX_SLICES = 4
+MS_QUERY_LAST_LAUNCHES = 5
 MS_ACT_NONE = 0
 MS_ACT_GELU = 1
 

@@ -61,6 +61,7 @@ int msi::fail(int code, const char *fmt, ...) {
 namespace {
 
 thread_local int g_variant = 0;
+thread_local int g_launches = 0;   // kernels launched by the last GEMM call of this thread
 
 using msi::fail;
 
@@ -198,6 +199,7 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
     if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, false, false, true, false>(gd, bd, stream, g);
     else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
   }
+  g_launches++;
   MS_HIP(hipGetLastError());
   return MS_OK;
 }
@@ -211,28 +213,30 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
 // ceil(tiles / CUs) rounds of one tile per CU, so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile reaches 1.06
 // with a k-contiguous A and 1.02 without, the 384x192 tile 1.04 and 1.0, 192-wide ring tiles about 0.93,
-// 128x128 tiles about 0.55).  The
-// ring-kernel defaults use four waves over two 64-deep stages when an operand is k-contiguous: whole
-// 128-byte lines per request, half as many barriers as 32-deep stages.
-int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
-  if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
-  int v = g_variant;
-  if (v == 0) {
-    struct Cand { int v, bm, bn; double eff; };
-    // with two m/n-contiguous operands (RS) the hand-scheduled tiles gain less over the 256x256 ring than with a
-    // k-contiguous operand, and the 192-wide ring tiles do best on four 32-deep stages
-    const bool rs = p.flow == RS;
-    const Cand cands[] = {{1, 256, 256, 1.0},                    {10, 256, 384, rs ? 1.02 : 1.06}, {11, 384, 192, rs ? 1.0 : 1.04},
-                          {rs ? 5 : 8, 256, 192, rs ? 0.95 : 0.93}, {rs ? 6 : 9, 192, 256, rs ? 0.95 : 0.93}, {3, 128, 128, 0.55}};
-    const long chunks = p.flow == OS ? 1 : p.S;
-    double best = 0;
-    for (const Cand &c : cands) {
-      const long tiles = (long)((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * chunks;
-      const long rounds = (tiles + dev.cus - 1) / dev.cus;
-      const double cost = (double)rounds * c.bm * c.bn / c.eff;
-      if (v == 0 || cost < best) { v = c.v; best = cost; }
-    }
+// 128x128 tiles about 0.55).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
+// k-contiguous: whole 128-byte lines per request, half as many barriers as 32-deep stages.
+struct Pick { int v; double cost; };
+
+// the single tile shape with the lowest estimated cost for the whole problem
+Pick pick_variant(const Problem &p, const DevInfo &dev) {
+  struct Cand { int v, bm, bn; double eff; };
+  // with two m/n-contiguous operands (RS) the hand-scheduled tiles gain less over the 256x256 ring than with a
+  // k-contiguous operand, and the 192-wide ring tiles do best on four 32-deep stages
+  const bool rs = p.flow == RS;
+  const Cand cands[] = {{1, 256, 256, 1.0},                    {10, 256, 384, rs ? 1.02 : 1.06}, {11, 384, 192, rs ? 1.0 : 1.04},
+                        {rs ? 5 : 8, 256, 192, rs ? 0.95 : 0.93}, {rs ? 6 : 9, 192, 256, rs ? 0.95 : 0.93}, {3, 128, 128, 0.55}};
+  const long chunks = p.flow == OS ? 1 : p.S;
+  Pick best = {0, 0};
+  for (const Cand &c : cands) {
+    const long tiles = (long)((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * chunks;
+    const long rounds = (tiles + dev.cus - 1) / dev.cus;
+    const double cost = (double)rounds * c.bm * c.bn / c.eff;
+    if (best.v == 0 || cost < best.cost) best = {c.v, cost};
   }
+  return best;
+}
+
+int launch_variant(int v, const Problem &p, const DevInfo &dev, hipStream_t stream) {
   switch (v) {
     case 1: return launch_bf16_tile<256, 256, 2, 2, 64, 2>(p, dev, stream);
     case 2: return launch_bf16_tile<256, 256, 2, 4, 32, 4>(p, dev, stream);
@@ -247,6 +251,50 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
     case 11: return launch_bf16_tile<384, 192, 2, 2, 64, 2, true>(p, dev, stream);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
+}
+
+// An output-stationary product whose best single tile shape leaves much of its last round idle is done in two
+// launches: the 256x384 tile on as many leading tile columns of C as fill whole rounds, the best shape for what
+// is left on the remaining columns (4096x9216x12288: 256 tiles of 256x384 plus 256 tiles of 256x192, 0.67 ms,
+// instead of 768 tiles of 256x192 in three rounds, 0.76 ms).  The second launch costs about a hundredth of a
+// millisecond (launch gap, one more prologue), which the estimate charges as tile area.  LS / RS are not split:
+// their chunks are promised in slice order.
+int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+  if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
+  if (g_variant != 0) return launch_variant(g_variant, p, dev, stream);
+  const Pick single = pick_variant(p, dev);
+  if (p.flow == OS) {
+    constexpr int BM = 256, BN = 384;
+    constexpr double EFF = 1.06;
+    const long tiles_m = (p.M + BM - 1) / BM;
+    const long total_k = (long)p.K * p.S;
+    // whole rounds of the big tile: the largest count of leading tile columns whose tiles are a multiple of the CUs
+    long nb1 = p.N / BN;
+    while (nb1 > 0 && (tiles_m * nb1) % dev.cus != 0) nb1--;
+    const long n1 = nb1 * BN;
+    if (nb1 > 0 && n1 < p.N) {
+      Problem rest = p;
+      rest.N = p.N - (int)n1;
+      const Pick tail = pick_variant(rest, dev);
+      const double second_launch = 3.4e7 / (double)total_k;      // ~12 us at the rate one CU computes tile area x K
+      const double cost = (double)(tiles_m * nb1 / dev.cus) * BM * BN / EFF + tail.cost + second_launch;
+      if (cost < 0.97 * single.cost) {
+        const int es_in = 2, es_out = p.out_dtype == MS_DTYPE_BF16 ? 2 : 4;
+        Problem head = p;
+        head.N = (int)n1;
+        int rc = launch_variant(10, head, dev, stream);
+        if (rc != MS_OK) return rc;
+        const void *b2[MS_MAX_SLICES];
+        void *c2[1] = {static_cast<char *>(p.c[0]) + n1 * es_out};
+        for (int s = 0; s < p.nb; s++) b2[s] = static_cast<const char *>(p.b[s]) + n1 * es_in;
+        rest.b = b2;
+        rest.c = c2;
+        if (p.res) rest.res = static_cast<const char *>(p.res) + n1 * es_out;
+        return launch_variant(tail.v, rest, dev, stream);
+      }
+    }
+  }
+  return launch_variant(single.v, p, dev, stream);
 }
 
 int launch_f32(const Problem &p, hipStream_t stream) {
@@ -270,6 +318,7 @@ int launch_f32(const Problem &p, hipStream_t stream) {
   dim3 gd((unsigned)total), bd(256);
   if (p.out_dtype == MS_DTYPE_BF16) hipLaunchKernelGGL(msk::gemm_f32_kernel<true>, gd, bd, 0, stream, g);
   else hipLaunchKernelGGL(msk::gemm_f32_kernel<false>, gd, bd, 0, stream, g);
+  g_launches++;
   MS_HIP(hipGetLastError());
   return MS_OK;
 }
@@ -281,6 +330,7 @@ int run(const Problem &p, void *stream) {
   rc = dev_info(&dev);
   if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
+  g_launches = 0;
   return p.in_dtype == MS_DTYPE_BF16 ? launch_bf16(p, *dev, st) : launch_f32(p, st);
 }
 
@@ -339,6 +389,7 @@ MS_API const char *ms_last_error(void) { return g_err; }
 
 MS_API long ms_query(int what) {
   if (what == MS_QUERY_MAX_SLICES) return MS_MAX_SLICES;
+  if (what == MS_QUERY_LAST_LAUNCHES) return g_launches;
   DevInfo *d = nullptr;
   if (dev_info(&d) != MS_OK) return -1;
   switch (what) {

@@ -88,3 +88,42 @@ def test_config4_rs_s4_full_size():
     for k in (0, 2):
         idx = torch.from_numpy(orc.sel(3072, 4, 8, k)).cuda()
         assert torch.equal(full[idx, :], Y[k])
+
+
+def test_os_with_a_fractional_last_round_is_split_into_two_launches():
+    """X[4096,12288] x W[12288,9216], S=4: no single tile shape fills its last round of compute units, so the call
+    runs the 256x384 tile on the first 6144 columns and the best shape for the rest on the other 3072.  The result
+    is the single-launch one (same products summed in the same order per element), with and without the fused
+    epilogue, for bf16 and fp32 outputs; the residual and the row moments follow the split."""
+    from meshslice_amd import _lib
+    L = _lib.load()
+    X = _randn_bf16((4096, 12288), 1.0, 40); W = _randn_bf16((12288, 9216), 0.02, 41)
+    A4, B4 = _slices_cols(X, 4), _slices_rows(W, 4)
+    for out_dtype in (torch.bfloat16, torch.float32):
+        L.ms_set_variant(0)
+        got = ms.gemm_os(A4, B4, out_dtype=out_dtype)
+        assert L.ms_query(_lib.MS_QUERY_LAST_LAUNCHES) == 2
+        L.ms_set_variant(8)
+        one = ms.gemm_os(A4, B4, out_dtype=out_dtype)
+        assert L.ms_query(_lib.MS_QUERY_LAST_LAUNCHES) == 1
+        L.ms_set_variant(0)
+        assert torch.equal(got, one)
+    rows = np.random.default_rng(3).choice(4096, 24, replace=False)
+    assert orc.rel_frobenius(_f64(got[rows]), _f64(X[rows]) @ _f64(W)) <= 1e-5 * 50    # fp32 out of bf16 operands
+    # fused epilogue through the split: GELU, a residual that spans both parts, row moments added by both launches
+    R = _randn_bf16((4096, 9216), 1.0, 42)
+    s1 = torch.zeros(4096, device="cuda"); s2 = torch.zeros(4096, device="cuda")
+    fused = ms.gemm_os(A4, B4, activation="gelu", residual=R, row_moments=(s1, s2))
+    assert L.ms_query(_lib.MS_QUERY_LAST_LAUNCHES) == 2
+    L.ms_set_variant(8)
+    t1 = torch.zeros(4096, device="cuda"); t2 = torch.zeros(4096, device="cuda")
+    fused_one = ms.gemm_os(A4, B4, activation="gelu", residual=R, row_moments=(t1, t2))
+    L.ms_set_variant(0)
+    assert torch.equal(fused, fused_one)
+    assert orc.rel_frobenius(_f64(s1), _f64(t1)) <= 1e-5 and orc.rel_frobenius(_f64(s2), _f64(t2)) <= 1e-5
+    want = torch.nn.functional.gelu(got.float(), approximate="tanh") + R.float()
+    assert orc.rel_frobenius(_f64(fused), _f64(want)) <= TOL_BF16
+    # a product that one shape covers in whole rounds stays one launch
+    ms.gemm_os(_slices_cols(X, 4), _slices_rows(_randn_bf16((12288, 12288), 0.02, 43), 4))
+    assert L.ms_query(_lib.MS_QUERY_LAST_LAUNCHES) == 1
+
