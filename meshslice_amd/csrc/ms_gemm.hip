@@ -212,7 +212,7 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
 // ceil(tiles / CUs) rounds of one tile per CU, so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile reaches 1.06
-// with a k-contiguous A and 1.02 without, the 384x192 tile 1.04 and 1.0, 192-wide ring tiles about 0.93,
+// with a k-contiguous A and 1.02 without, the 384x192 tile 1.04 and 0.96, 192-wide ring tiles about 0.93,
 // 128x128 tiles about 0.55).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
 // k-contiguous: whole 128-byte lines per request, half as many barriers as 32-deep stages.
 struct Pick { int v; double cost; };
@@ -223,7 +223,7 @@ Pick pick_variant(const Problem &p, const DevInfo &dev) {
   // with two m/n-contiguous operands (RS) the hand-scheduled tiles gain less over the 256x256 ring than with a
   // k-contiguous operand, and the 192-wide ring tiles do best on four 32-deep stages
   const bool rs = p.flow == RS;
-  const Cand cands[] = {{1, 256, 256, 1.0},                    {10, 256, 384, rs ? 1.02 : 1.06}, {11, 384, 192, rs ? 1.0 : 1.04},
+  const Cand cands[] = {{1, 256, 256, 1.0},                    {10, 256, 384, rs ? 1.02 : 1.06}, {11, 384, 192, rs ? 0.96 : 1.04},
                         {rs ? 5 : 8, 256, 192, rs ? 0.95 : 0.93}, {rs ? 6 : 9, 192, 256, rs ? 0.95 : 0.93}, {3, 128, 128, 0.55}};
   const long chunks = p.flow == OS ? 1 : p.S;
   Pick best = {0, 0};
