@@ -23,9 +23,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6     # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
 # Bytes per launch of the config-2 kernel that cross the L2 <-> fabric boundary (Infinity Cache or HBM), from
-# two rocprofv3 --pmc runs (FETCH_SIZE 700104 KiB-units x 2.0 and WRITE_SIZE 114176 x 1.0, each scaled by what
+# two rocprofv3 --pmc runs (FETCH_SIZE 692250 KiB-units x 2.0 and WRITE_SIZE 104960 x 1.0, each scaled by what
 # the same counter reads for a 1 GiB device copy in the same run); summary in profiles/gemm_bf16_big_256x384x64_os_cfg2.md.
-MEASURED_TRAFFIC_BYTES = 1550649912
+MEASURED_TRAFFIC_BYTES = 1525127376
 
 
 def sel_index(L, S, B, k):
