@@ -123,6 +123,19 @@ def test_os_with_a_fractional_last_round_is_split_into_two_launches():
     assert orc.rel_frobenius(_f64(s1), _f64(t1)) <= 1e-5 and orc.rel_frobenius(_f64(s2), _f64(t2)) <= 1e-5
     want = torch.nn.functional.gelu(got.float(), approximate="tanh") + R.float()
     assert orc.rel_frobenius(_f64(fused), _f64(want)) <= TOL_BF16
+    # both launches are recorded when the call is captured in a HIP graph
+    out = torch.empty((4096, 9216), dtype=torch.bfloat16, device="cuda")
+    ms.gemm_os(A4, B4, out=out)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ms.gemm_os(A4, B4, out=out)
+    for _ in range(2):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ms.gemm_os(A4, B4))
     # a product that one shape covers in whole rounds stays one launch
     ms.gemm_os(_slices_cols(X, 4), _slices_rows(_randn_bf16((12288, 12288), 0.02, 43), 4))
     assert L.ms_query(_lib.MS_QUERY_LAST_LAUNCHES) == 1
