@@ -59,7 +59,8 @@ long ms_query(int what);
  * Replaces the contractions of MeshFlow_OS (reference TensorParallel.py:162,167,172); with S == 1
  * it is Collective_OS (TensorParallel.py:22).  A_s is the s-th all-gathered column slice of the
  * activations (lda), B_s the s-th all-gathered row slice of the weights (ldb).  C is written in
- * out_dtype (ldc). */
+ * out_dtype (ldc).  A call is one kernel launch on `stream`, or two (disjoint column ranges of C) when one
+ * tile shape alone would leave much of its last round of compute units idle. */
 int ms_gemm_os(const void *const *A_slices, const void *const *B_slices, int S,
                int m, int n, int k_slice, int lda, int ldb,
                void *C, int ldc, int in_dtype, int out_dtype, void *stream);
