@@ -195,6 +195,10 @@ def main():
         extra["os_s4_fused_gelu_ms"] = round(_events(lambda: ms.gemm_os(A, B, out=C, activation="gelu"), 10), 4)
         extra["os_s4_then_separate_gelu_ms"] = round(_events(
             lambda: torch.nn.functional.gelu(ms.gemm_os(A, B, out=C), approximate="tanh"), 10), 4)
+        # the vendor library's GEMM (hipBLASLt through torch.matmul) on the same un-sliced operands, same box, for scale
+        torch.matmul(X, W)
+        extra["vendor_library_matmul_s1_ms"] = round(_events(lambda: torch.matmul(X, W), 30), 4)
+        extra["os_s1_same_method_ms"] = round(_events(lambda: ms.gemm_os([X], [W], out=C), 30), 4)
         # the layout kernels either side of the GEMM on the same [4096, 12288] bf16 shard: algorithmic GB/s (HBM roofline 8000)
         from meshslice_amd.slice_layout import measure_rates
         for label, t, nbytes in measure_rates(dtypes=(torch.bfloat16,), reduce_case=False, reps=24):
