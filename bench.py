@@ -204,6 +204,18 @@ def main():
         for label, t, nbytes in measure_rates(dtypes=(torch.bfloat16,), reduce_case=False, reps=24):
             key = "layout_" + label.replace("bfloat16 ", "").replace(" of the shard", "").replace("=", "").replace(" ", "_").lower() + "_gbps"
             extra[key] = round(nbytes / t / 1e9, 0)
+        # one device's whole output-stationary step on a 4x4 mesh: cut its own X shard [4096, 3072] and W shard [3072, 12288]
+        # into the S slices it sends to its peers (the peers' slices arrive by all-gather), then the sliced GEMM
+        from meshslice_amd.slice_layout import pack_slices
+        Xown, Wown = X[:, :K // 4].contiguous(), W[:K // 4, :].contiguous()
+        xs = pack_slices(Xown, S, 8, 1); ws = pack_slices(Wown, S, 8, 0)
+
+        def _device_step():
+            pack_slices(Xown, S, 8, 1, out=xs)
+            pack_slices(Wown, S, 8, 0, out=ws)
+            ms.gemm_os(A, B, out=C)
+        extra["os_s4_device_step_ms"] = round(_events(_device_step, 20), 4)
+        extra["os_s4_gemm_alone_same_method_ms"] = round(_events(lambda: ms.gemm_os(A, B, out=C), 20), 4)
         # what this device sustains on the bare MFMA instruction stream (no memory traffic) for operands drawn
         # like X: the practical, power-limited ceiling beside the data-sheet peak
         from meshslice_amd.local_gemm import mfma_stream_rate
