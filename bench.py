@@ -219,7 +219,7 @@ def main():
         # what this device sustains on the bare MFMA instruction stream (no memory traffic) for operands drawn
         # like X: the practical, power-limited ceiling beside the data-sheet peak
         from meshslice_amd.local_gemm import mfma_stream_rate
-        stream_tf = mfma_stream_rate(X[:8, :512].contiguous().reshape(-1)) / 1e12
+        stream_tf = mfma_stream_rate(X[:16, :512].contiguous().reshape(-1)) / 1e12
         extra["mfma_stream_ceiling_tflops"] = round(stream_tf, 1)
         extra["achieved_over_mfma_stream_ceiling"] = round(value / stream_tf, 4)
 

@@ -130,6 +130,15 @@ int ms_time_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int
                int m_slice, int n, int k,
                float *const *Y_chunks, int ldy, int in_dtype, void *stream,
                int warmup, int reps, float *ms_out);
+/* The same for ms_gemm_ls_ex / ms_gemm_rs_ex (chunks in out_dtype). */
+int ms_time_ls_ex(const void *A, int lda, const void *const *W_slices, int ldw, int S,
+                  int m, int n_slice, int k,
+                  void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream,
+                  int warmup, int reps, float *ms_out);
+int ms_time_rs_ex(const void *const *X_slices, int ldx, const void *W, int ldw, int S,
+                  int m_slice, int n, int k,
+                  void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream,
+                  int warmup, int reps, float *ms_out);
 
 /* Block-cyclic slices of a shard, all S of them in one pass over it:
  *     axis 1:  dst_slices[s][r, (b / S) * B + e] = src[r, b * B + e]   for column blocks b with b % S == s
@@ -160,14 +169,23 @@ int ms_unpack_chunks(const void *const *chunks, int P, int S, int ld_chunk, int 
                      int in_dtype, int out_dtype, void *stream);
 
 /* Measurement aid (no counterpart in the reference): the rate at which the current device sustains a bare
- * stream of v_mfma_f32_32x32x16_bf16, the instruction the bf16 kernels are built on — one wave per SIMD,
- * operands and accumulators resident in registers, no memory traffic.  Under its package power limit the
- * device clocks this stream below the data-sheet frequency, by an amount that depends on the operand
- * data, so this is the practical ceiling against which a kernel's achieved rate can be read.
- * operands: 8 fragments x 64 lanes x 8 bf16 (8 KB, 16-byte aligned), typically the same distribution as
- * the GEMM's inputs; sink: one float per launched thread (256 x CU count floats) that receives the sums;
- * iters: loop trips of 64 MFMAs per wave.  Launches warmup + reps kernels on `stream`, waits, and
- * returns the mean milliseconds per launch in *ms_out and the FLOPs of one launch in *flops_per_launch. */
+ * stream of one bf16 MFMA instruction — operands and accumulators resident in registers, no memory traffic.
+ * Under its package power limit the device clocks such a stream below the data-sheet frequency, by an amount
+ * that depends on the instruction, on the waves per SIMD that issue it and on the operand data, so this is
+ * the practical ceiling against which a kernel's achieved rate can be read.
+ * shape: MS_MFMA_32X32X16 (v_mfma_f32_32x32x16_bf16, 8 passes) or MS_MFMA_16X16X32 (v_mfma_f32_16x16x32_bf16,
+ * 4 passes); waves_per_simd: 1 or 2 (workgroups of 4 or 8 waves, one per compute unit).
+ * operands: 16 fragments x 64 lanes x 8 bf16 (16 KB, 16-byte aligned), typically drawn like the GEMM's inputs;
+ * sink: one float per launched thread (256 x waves_per_simd x CU count floats) that receives the sums;
+ * iters: loop trips of 64 MFMAs per wave.  Launches warmup + reps kernels on `stream`, waits, and returns the
+ * mean milliseconds per launch in *ms_out and the FLOPs of one launch in *flops_per_launch. */
+#define MS_MFMA_32X32X16 0
+#define MS_MFMA_16X16X32 1
+int ms_probe_mfma_stream_ex(const void *operands, float *sink, int shape, int waves_per_simd, int iters,
+                            int warmup, int reps, float *ms_out, double *flops_per_launch, void *stream);
+
+/* ms_probe_mfma_stream_ex for MS_MFMA_32X32X16 at one wave per SIMD, the instruction and occupancy of the
+ * big-tile bf16 kernels; reads the first 8 fragments (8 KB) of operands. */
 int ms_probe_mfma_stream(const void *operands, float *sink, int iters, int warmup, int reps,
                          float *ms_out, double *flops_per_launch, void *stream);
 

@@ -3,7 +3,9 @@
 * ``FFLayerModel`` with its dataflow rule and ``emulate`` (reference Autotuner.py:21-35, :141-169):
   forward + backward-data + backward-weight model time of one feed-forward layer for a slice count;
 * ``possibleK`` (:242-273): admissible slice counts from the divisibility of the sliced extent;
-* ``emulateFFTime`` (:391-426): per layer, scan the candidate slice counts and keep the best;
+* ``emulateFFTime`` (:391-426): per layer, scan the candidate slice counts and keep the best — as the method
+  of ``class Autotuner(graph, shapes)`` like the reference's (same name, arguments and return value), and as
+  a free function over a plain layer list;
 * the interconnect constants the reference measured on TPUv4 (:17-19), kept as data;
 * ``sweep_compute_term``: time the per-slice kernels of one GPT-3-like layer on the MI355X for
   several meshes and slice counts and refit ``CostModel.estimateMatmul``'s compute term.
@@ -112,6 +114,131 @@ def emulateFFTime(layers: Sequence[Tuple[int, int, int, str]], meshshape, sweep:
     return total, best
 
 
+class LayerGraph:
+    """The two attributes of the reference's ``ComputeGraph`` that its ``Autotuner`` reads (``nodenames`` and
+    ``nodes``, reference :171-223), built from a list of feed-forward layers ``(name, B, I, O)``: each layer
+    becomes an 'Input' node of shape [B, I] feeding a 'FeedForward' node of shape [B, O]."""
+
+    def __init__(self, layers: Iterable[Tuple[str, int, int, int]]):
+        self.nodenames: List[str] = []
+        self.nodes: Dict[str, dict] = {}
+        for (name, B, I, O) in layers:
+            src = f"Input:{name}"
+            for nm, op, inputs, shape in ((src, "Input", (), [B, I]), (name, "FeedForward", (src,), [B, O])):
+                self.nodenames.append(nm)
+                self.nodes[nm] = {"op_name": nm, "op_type": op, "inputs": inputs, "shape": shape}
+
+
+class Autotuner:
+    """The slice-count / mesh-shape search of the reference's ``Autotuner`` that runs on the measured compute
+    term (reference Autotuner.py:278-483): ``emulateFFTime(meshshape, sweep)`` and ``emulatedFinetune(sweep)``.
+
+    ``graph`` is anything with the reference ``ComputeGraph``'s ``nodenames`` / ``nodes`` (a ``LayerGraph``
+    built from a layer list will do); ``shapes`` the candidate mesh shapes, all with the same device count.
+    Per feed-forward node the dataflow follows the reference's rule (:291-302) and an 'rs' layer flips the
+    transposition of what follows it (:303-313).  Not built: the analytical first guess (``analyticalAutotune``,
+    host arithmetic on link constants) — the search starts from ``bestshape`` (default ``shapes[0]``) — and the
+    insertion of 'Transpose' nodes where the two inputs of an 'Add' disagree (the 'Add' is taken as not
+    transposed).  ``emulateFFTime`` records the loop variable as a layer's best slice count where the
+    reference stores its module-level ``K`` (:418); ``emulatedFinetune(sweep=True)`` keeps the best shape where
+    the reference assigns a misspelt attribute and returns nothing (:440)."""
+
+    def __init__(self, graph, shapes, bestshape=None, verbose: bool = False):
+        self.graph = graph
+        self.shapes = list(shapes)
+        self.layers = list(graph.nodenames)
+        self.verbose = verbose
+        self.dataflows: Dict[str, str] = {}
+        self.transposition: Dict[str, bool] = {}
+        self.ksplits: Dict[str, int] = {}
+        for lname in self.layers:
+            node = graph.nodes[lname]
+            if node["op_type"] == "FeedForward":
+                self.dataflows[lname] = pick_dataflow(*self._dims(lname))
+        for lname in self.layers:
+            node = graph.nodes[lname]
+            if node["op_type"] == "Input":
+                self.transposition[lname] = False
+            elif node["op_type"] == "Add":
+                a, b = (self.transposition[i] for i in node["inputs"][:2])
+                self.transposition[lname] = a and b
+            else:
+                t = self.transposition[node["inputs"][0]]
+                self.transposition[lname] = (not t) if self.dataflows.get(lname) == "rs" else t
+        self.bestshape = tuple(bestshape) if bestshape is not None else tuple(self.shapes[0])
+        if self.bestshape not in [tuple(s) for s in self.shapes]:
+            raise ValueError(f"bestshape {self.bestshape} is not one of the candidate shapes")
+
+    def _dims(self, lname) -> Tuple[int, int, int]:
+        """(B, I, O) of feed-forward node ``lname``: B = product of the leading output dimensions, I = last
+        dimension of its input, O = last dimension of its output (reference :292-297)."""
+        node = self.graph.nodes[lname]
+        B = 1
+        for d in node["shape"][:-1]:
+            B *= d
+        return B, self.graph.nodes[node["inputs"][0]]["shape"][-1], node["shape"][-1]
+
+    def _say(self, msg: str) -> None:
+        if self.verbose:
+            print(msg)
+
+    def emulateFFTime(self, meshshape, sweep: bool = False):
+        """Model seconds of all feed-forward nodes on ``meshshape`` with each node's best slice count, and those
+        counts by node name (reference :391-426).  Without ``sweep`` a node's scan over ``possibleK`` stops at
+        the first count that does not improve."""
+        mesh = default_mesh(tuple(meshshape), flops=242 * 1024 ** 4)
+        total, ksplits = 0.0, {}
+        for lname in self.graph.nodenames:
+            if self.graph.nodes[lname]["op_type"] != "FeedForward":
+                continue
+            B, I, O = self._dims(lname)
+            model = FFLayerModel(B, I, O, self.dataflows[lname], self.transposition[lname])
+            klist = possibleK(B, I, O, meshshape, self.dataflows[lname])
+            bestK, bestT = klist[0], model.emulate(mesh, klist[0])
+            self._say(f"{lname}: candidates {klist}; FFtime at k={bestK} is {bestT}")
+            for k in klist[1:]:
+                t = model.emulate(mesh, k)
+                self._say(f"FFtime at k={k} is {t}")
+                if t < bestT:
+                    bestK, bestT = k, t
+                elif not sweep:
+                    break
+            total += bestT
+            ksplits[lname] = bestK
+        self._say(f"FFtime: {total * 1000}ms")
+        return total, ksplits
+
+    def emulatedFinetune(self, sweep: bool = False):
+        """Walk from ``bestshape`` to a neighbouring mesh shape while the model time drops (reference :427-483);
+        with ``sweep`` try every shape.  Sets and returns ``(bestshape, ksplits)``."""
+        times = {}
+
+        def at(idx):
+            if idx not in times:
+                self._say(f"Trying shape of {self.shapes[idx]}")
+                times[idx] = self.emulateFFTime(self.shapes[idx], sweep=sweep)
+            return times[idx]
+
+        shapes = [tuple(s) for s in self.shapes]
+        cur = shapes.index(self.bestshape)
+        if sweep:
+            best = min(range(len(shapes)), key=lambda i: (at(i)[0], i != cur))
+        else:
+            def walk(idx, step):
+                while 0 <= idx + step < len(shapes) and at(idx + step)[0] < at(idx)[0]:
+                    idx += step
+                return idx
+            if cur > 0 and at(cur - 1)[0] < at(cur)[0]:          # the previous shape first, as the reference
+                best = walk(cur - 1, -1)
+            elif cur + 1 < len(shapes) and at(cur + 1)[0] < at(cur)[0]:
+                best = walk(cur + 1, +1)
+            else:
+                best = cur
+        self.bestshape, self.ksplits = shapes[best], at(best)[1]
+        self._say(f"Best mesh shape is : {self.bestshape}")
+        return self.bestshape, self.ksplits
+
+
 # ------------------------------------------------------------------------------------------------
 # compute-term sweep on the MI355X
 # ------------------------------------------------------------------------------------------------
@@ -142,8 +269,10 @@ def per_slice_shapes(B, I, O, dataflow, meshshape, S, passes=("fwd", "bwd_data",
 
 
 def sweep_compute_term(meshes=((2, 8), (4, 4), (8, 8)), slice_counts=(1, 2, 4, 8, 16),
-                       passes=("fwd",), layers=None, repeat: int = 5, verbose: bool = True, fused: bool = False):
-    """Measure every per-slice kernel of the sweep on the GPU and fit the compute term.
+                       passes=("fwd",), layers=None, repeat: int = 5, verbose: bool = True, fused: bool = False,
+                       operands=None):
+    """Measure every per-slice kernel of the sweep on the GPU and fit the compute term.  ``operands`` ('normal' or
+    'ones', default CostModel.DEFAULT_OPERANDS) says what the timing operands hold, see CostModel.estimateMatmul.
 
     Returns ``(ComputeTerm, rows)`` where each row is
     ``(mesh, layer, pass, S, M, N, K, layout, seconds_per_slice)``; with ``fused`` a tenth entry holds the
@@ -156,14 +285,14 @@ def sweep_compute_term(meshes=((2, 8), (4, 4), (8, 8)), slice_counts=(1, 2, 4, 8
                 for (pname, M, N, K, layout) in per_slice_shapes(B, I, O, dataflow, mesh, S, passes):
                     key = (M, N, K, layout)
                     if key not in seen:
-                        seen[key] = CostModel.estimateMatmul(None, M, N, K, layout=layout, repeat=repeat)
+                        seen[key] = CostModel.estimateMatmul(None, M, N, K, layout=layout, repeat=repeat, operands=operands)
                         samples.append((M, N, K, layout, seen[key]))
                     row = (mesh, lname, pname, S, M, N, K, layout, seen[key])
                     extra = ""
                     if fused:
                         fk = key + (S,)
                         if fk not in seen_fused:
-                            seen_fused[fk] = CostModel.measureFused(M, N, K, S, layout=layout, repeat=repeat)
+                            seen_fused[fk] = CostModel.measureFused(M, N, K, S, layout=layout, repeat=repeat, operands=operands)
                         row = row + (seen_fused[fk],)
                         ftf = 2.0 * M * N * K * S / seen_fused[fk] / 1e12
                         extra = f" | S x slice {S*seen[key]*1e3:.4f} ms, fused {seen_fused[fk]*1e3:.4f} ms {ftf:.0f} TFLOP/s"
@@ -186,11 +315,13 @@ def _main(argv=None):
     ap.add_argument("--meshes", default="2x8,4x4,8x8")
     ap.add_argument("--repeat", type=int, default=5)
     ap.add_argument("--fused", action="store_true", help="also time the fused S-slice call of every row")
+    ap.add_argument("--operands", default=CostModel.DEFAULT_OPERANDS, choices=CostModel.OPERAND_KINDS,
+                    help="timing operands: N(0, 0.02) samples, or all ones as in the reference")
     ap.add_argument("--out", default=None, help="write the fitted term and the rows as JSON")
     a = ap.parse_args(argv)
     meshes = [tuple(int(v) for v in m.split("x")) for m in a.meshes.split(",")]
     slices = [int(v) for v in a.slices.split(",")]
-    term, rows = sweep_compute_term(meshes, slices, tuple(a.passes.split(",")), repeat=a.repeat, fused=a.fused)
+    term, rows = sweep_compute_term(meshes, slices, tuple(a.passes.split(",")), repeat=a.repeat, fused=a.fused, operands=a.operands)
     for lay in sorted(term.eta):
         print(f"fit {lay}: t0 = {term.t0[lay]*1e6:.1f} us, eta = {term.eta[lay]:.3f} of {term.peak/1e12:.1f} TFLOP/s")
     CostModel.use_compute_term(term)
@@ -204,7 +335,9 @@ def _main(argv=None):
         CostModel.use_compute_term(None)
     if a.out:
         with open(a.out, "w") as f:
-            json.dump({"term": term.to_dict(),
+            what = "N(0, 0.02) samples" if a.operands == "normal" else "ones as in the reference's estimateMatmul"
+            json.dump({"device": f"MI355X (gfx950), bf16, operands filled with {what}", "operands": a.operands,
+                       "term": term.to_dict(),
                        "rows": [[f"{r[0][0]}x{r[0][1]}"] + list(r[1:]) for r in rows]}, f, indent=1)
 
 

@@ -7,7 +7,8 @@ seconds.  The SUMMA / Cannon / logical-ring models of the reference are comparis
 not built.
 
 The compute term is what this build changes: ``estimateMatmul`` times the gfx950 kernel of the same
-layout on the MI355X (HIP events, one warm-up + ``repeat`` launches, mean), or — when a fitted
+layout on the MI355X (HIP events, warm-up + ``repeat`` launches, mean; operands N(0, 0.02) by default, all ones
+as in the reference on request), or — when a fitted
 ``ComputeTerm`` has been installed with ``use_compute_term`` — evaluates ``t0 + 2MNK / (eta * peak)``
 without touching the GPU.  There is no CPU timing path.
 """
@@ -139,13 +140,29 @@ def use_compute_term(term: Optional[ComputeTerm]) -> None:
     _installed = term
 
 
-def load_compute_term(path: Optional[str] = None) -> ComputeTerm:
-    """Install the compute term measured on MI355X that ships with the package (or the JSON at ``path``,
-    as written by ``python -m meshslice_amd.Autotuner --out``) and return it."""
-    import json
+OPERAND_KINDS = ("normal", "ones")
+# What the timing operands hold when a call does not say: N(0, 0.02) values rounded to bf16.  The reference times
+# its matmul on all-ones operands (CostModel.py:78-79); on this power-limited device constant operands run
+# 20-25 % faster than real tensors, which would bias the compute term low against every communication term.
+DEFAULT_OPERANDS = "normal"
+# untimed launches before the timed ones: one for 'ones' (the reference's protocol, :90); for 'normal' enough to
+# pass the start-up transient of the package power controller, during which launches run up to 30 % slow
+_WARMUP = {"ones": 1, "normal": 10}
+
+
+def _term_path(operands: str) -> str:
     import os
+    name = "compute_term_mi355x.json" if operands == "normal" else "compute_term_mi355x_ones.json"
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "data", name)
+
+
+def load_compute_term(path: Optional[str] = None, operands: Optional[str] = None) -> ComputeTerm:
+    """Install a compute term measured on MI355X that ships with the package and return it: by default the
+    one fitted on N(0, 0.02) operands, with ``operands='ones'`` the one fitted on the reference's all-ones
+    timing operands.  ``path`` names another JSON as written by ``python -m meshslice_amd.Autotuner --out``."""
+    import json
     if path is None:
-        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "data", "compute_term_mi355x.json")
+        path = _term_path(_operand_kind(operands))
     with open(path) as f:
         d = json.load(f)
     term = ComputeTerm.from_dict(d["term"] if "term" in d else d)
@@ -153,67 +170,82 @@ def load_compute_term(path: Optional[str] = None) -> ComputeTerm:
     return term
 
 
-def estimateMatmul(mesh, M, N, K, input_precision=None, layout: str = "nn", repeat: int = 5) -> float:
+def _operand_kind(operands: Optional[str]) -> str:
+    kind = DEFAULT_OPERANDS if operands is None else operands
+    if kind not in OPERAND_KINDS:
+        raise ValueError(f"unknown operand kind {kind!r} (one of {OPERAND_KINDS})")
+    return kind
+
+
+def _timing_operand(shape, dtype, kind: str, seed: int):
+    """A [rows, cols] GPU tensor of ones, or of seeded N(0, 0.02) samples rounded to ``dtype``."""
+    import torch
+    if kind == "ones":
+        return torch.ones(shape, dtype=dtype, device="cuda")
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (torch.randn(shape, generator=g, device="cuda") * 0.02).to(dtype)
+
+
+def _time_layout(M, N, K, S, layout, dtype, kind, repeat):
+    """Mean seconds per launch of the fused S-slice call of ``layout`` on per-slice shape [M,K] x [K,N]."""
+    import torch
+    from . import local_gemm
+    mk = lambda shape, i: _timing_operand(shape, dtype, kind, 1 + i)
+    warm = _WARMUP[kind]
+    if layout == "nn":
+        A = [mk((M, K), 2 * s) for s in range(S)]; B = [mk((K, N), 2 * s + 1) for s in range(S)]
+        ms = local_gemm.time_call("os", (A, B), torch.empty((M, N), dtype=dtype, device="cuda"), warmup=warm, reps=repeat)
+    elif layout == "nt":
+        out = [torch.empty((M, N), dtype=torch.float32, device="cuda") for _ in range(S)]
+        ms = local_gemm.time_call("ls", (mk((M, K), 0), [mk((N, K), 1 + s) for s in range(S)]), out, warmup=warm, reps=repeat)
+    else:
+        out = [torch.empty((M, N), dtype=torch.float32, device="cuda") for _ in range(S)]
+        ms = local_gemm.time_call("rs", ([mk((K, M), 1 + s) for s in range(S)], mk((K, N), 0)), out, warmup=warm, reps=repeat)
+    return float(np.mean(ms)) * 1e-3
+
+
+def estimateMatmul(mesh, M, N, K, input_precision=None, layout: str = "nn", repeat: int = 5,
+                   operands: Optional[str] = None) -> float:
     """Seconds of one local ``[M,K] x [K,N]`` contraction (reference CostModel.py:74-98).
 
     ``layout``: 'nn' (OS slice), 'nt' (LS: B stored [N,K]), 'tn' (RS: A stored [K,M]).  ``mesh`` is
-    unused, as in the reference.  Measures on the GPU unless a fitted term is installed."""
+    unused, as in the reference.  Measures on the GPU unless a fitted term is installed: ``operands='ones'``
+    is the reference's protocol (all-ones operands, one warm-up launch), ``'normal'`` (the default, see
+    DEFAULT_OPERANDS) times N(0, 0.02) operands after ten warm-up launches."""
     if layout not in ("nn", "nt", "tn"):
         raise ValueError(f"unknown layout {layout!r}")
+    kind = _operand_kind(operands)
     M, N, K = int(M), int(N), int(K)
     if _installed is not None:
         return _installed.seconds(M, N, K, layout)
     import torch
     from . import local_gemm
     dtype = input_precision or torch.bfloat16
-    key = (M, N, K, layout, dtype, repeat)
+    key = (M, N, K, layout, dtype, repeat, kind)
     if key in _measured:
         return _measured[key]
     if not torch.cuda.is_available():
         raise local_gemm._lib.MeshSliceError(
             "estimateMatmul needs the GPU (or a fitted ComputeTerm installed with use_compute_term)")
-    dev = "cuda"
-    if layout == "nn":
-        A = torch.ones((M, K), dtype=dtype, device=dev); B = torch.ones((K, N), dtype=dtype, device=dev)
-        out = torch.empty((M, N), dtype=dtype, device=dev)
-        ms = local_gemm.time_call("os", ([A], [B]), out, warmup=1, reps=repeat)
-    elif layout == "nt":
-        A = torch.ones((M, K), dtype=dtype, device=dev); B = torch.ones((N, K), dtype=dtype, device=dev)
-        out = [torch.empty((M, N), dtype=torch.float32, device=dev)]
-        ms = local_gemm.time_call("ls", (A, [B]), out, warmup=1, reps=repeat)
-    else:
-        A = torch.ones((K, M), dtype=dtype, device=dev); B = torch.ones((K, N), dtype=dtype, device=dev)
-        out = [torch.empty((M, N), dtype=torch.float32, device=dev)]
-        ms = local_gemm.time_call("rs", ([A], B), out, warmup=1, reps=repeat)
-    sec = float(np.mean(ms)) * 1e-3
+    sec = _time_layout(M, N, K, 1, layout, dtype, kind, repeat)
     _measured[key] = sec
     return sec
 
 
-def measureFused(M, N, K, S, layout: str = "nn", input_precision=None, repeat: int = 5) -> float:
+def measureFused(M, N, K, S, layout: str = "nn", input_precision=None, repeat: int = 5,
+                 operands: Optional[str] = None) -> float:
     """Seconds of ONE fused call that does the work of ``S`` per-slice contractions of shape
     ``[M,K] x [K,N]`` (the per-slice shape ``estimateMatmul`` is asked about): 'nn' = ms_gemm_os over S
-    k-slices, 'nt' = ms_gemm_ls emitting S chunks, 'tn' = ms_gemm_rs emitting S chunks.  GPU only."""
+    k-slices, 'nt' = ms_gemm_ls emitting S chunks, 'tn' = ms_gemm_rs emitting S chunks.  GPU only;
+    ``operands`` as in ``estimateMatmul``."""
     import torch
     from . import local_gemm
     if layout not in ("nn", "nt", "tn"):
         raise ValueError(f"unknown layout {layout!r}")
+    kind = _operand_kind(operands)
     if not torch.cuda.is_available():
         raise local_gemm._lib.MeshSliceError("measureFused needs the GPU")
-    dtype = input_precision or torch.bfloat16
-    M, N, K, S = int(M), int(N), int(K), int(S)
-    dev = "cuda"
-    ones = lambda *shape: torch.ones(shape, dtype=dtype, device=dev)
-    if layout == "nn":
-        A = [ones(M, K) for _ in range(S)]; B = [ones(K, N) for _ in range(S)]
-        ms = local_gemm.time_call("os", (A, B), torch.empty((M, N), dtype=dtype, device=dev), warmup=1, reps=repeat)
-    elif layout == "nt":
-        out = [torch.empty((M, N), dtype=torch.float32, device=dev) for _ in range(S)]
-        ms = local_gemm.time_call("ls", (ones(M, K), [ones(N, K) for _ in range(S)]), out, warmup=1, reps=repeat)
-    else:
-        out = [torch.empty((M, N), dtype=torch.float32, device=dev) for _ in range(S)]
-        ms = local_gemm.time_call("rs", ([ones(K, M) for _ in range(S)], ones(K, N)), out, warmup=1, reps=repeat)
-    return float(np.mean(ms)) * 1e-3
+    return _time_layout(int(M), int(N), int(K), int(S), layout, input_precision or torch.bfloat16, kind, repeat)
 
 
 # ------------------------------------------------------------------------------------------------

@@ -24,6 +24,8 @@ MS_QUERY_MAX_SLICES = 4
 MS_QUERY_LAST_LAUNCHES = 5
 MS_ACT_NONE = 0
 MS_ACT_GELU = 1
+MS_MFMA_32X32X16 = 0
+MS_MFMA_16X16X32 = 1
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmeshslice_hip.so")
@@ -31,8 +33,8 @@ LIB_PATH = os.path.join(_HERE, "libmeshslice_hip.so")
 EXPORTS = (
     "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
     "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex",
-    "ms_time_os", "ms_time_ls", "ms_time_rs",
-    "ms_pack_slices", "ms_unpack_chunks", "ms_probe_mfma_stream",
+    "ms_time_os", "ms_time_ls", "ms_time_rs", "ms_time_ls_ex", "ms_time_rs_ex",
+    "ms_pack_slices", "ms_unpack_chunks", "ms_probe_mfma_stream", "ms_probe_mfma_stream_ex",
 )
 
 _lock = threading.Lock()
@@ -68,6 +70,8 @@ def _declare(lib):
     lib.ms_time_os.argtypes = os_args + [c_int, c_int, fp]
     lib.ms_time_ls.argtypes = ls_args + [c_int, c_int, fp]
     lib.ms_time_rs.argtypes = rs_args + [c_int, c_int, fp]
+    lib.ms_time_ls_ex.argtypes = ls_args[:-1] + [c_int, c_vp, c_int, c_int, fp]    # ..., in_dtype, out_dtype, stream, warmup, reps, ms_out
+    lib.ms_time_rs_ex.argtypes = rs_args[:-1] + [c_int, c_vp, c_int, c_int, fp]
     # src, ld_src, rows, cols, axis, S, B, dst_slices, ld_dst, dtype, stream
     lib.ms_pack_slices.argtypes = [c_vp, c_int, c_int, c_int, c_int, c_int, c_int, vpp, c_int, c_int, c_vp]
     lib.ms_pack_slices.restype = c_int
@@ -77,7 +81,11 @@ def _declare(lib):
     # operands, sink, iters, warmup, reps, ms_out, flops_per_launch, stream
     lib.ms_probe_mfma_stream.argtypes = [c_vp, c_vp, c_int, c_int, c_int, fp, ctypes.POINTER(ctypes.c_double), c_vp]
     lib.ms_probe_mfma_stream.restype = c_int
-    for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_time_os", "ms_time_ls", "ms_time_rs"):
+    # operands, sink, shape, waves_per_simd, iters, warmup, reps, ms_out, flops_per_launch, stream
+    lib.ms_probe_mfma_stream_ex.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, fp, ctypes.POINTER(ctypes.c_double), c_vp]
+    lib.ms_probe_mfma_stream_ex.restype = c_int
+    for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_time_os", "ms_time_ls", "ms_time_rs",
+              "ms_time_ls_ex", "ms_time_rs_ex"):
         getattr(lib, n).restype = c_int
 
 

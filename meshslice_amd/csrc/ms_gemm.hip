@@ -453,14 +453,26 @@ MS_API int ms_time_os(const void *const *A_slices, const void *const *B_slices, 
   return timed(make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype), stream, warmup, reps, ms_out);
 }
 
+MS_API int ms_time_ls_ex(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
+                         void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream,
+                         int warmup, int reps, float *ms_out) {
+  const void *a1[1] = {A};
+  return timed(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, Y_chunks, ldy, in_dtype, out_dtype), stream, warmup, reps, ms_out);
+}
+
+MS_API int ms_time_rs_ex(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
+                         void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream,
+                         int warmup, int reps, float *ms_out) {
+  const void *w1[1] = {W};
+  return timed(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype, out_dtype), stream, warmup, reps, ms_out);
+}
+
 MS_API int ms_time_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
                       float *const *Y_chunks, int ldy, int in_dtype, void *stream, int warmup, int reps, float *ms_out) {
-  const void *a1[1] = {A};
-  return timed(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, (void *const *)Y_chunks, ldy, in_dtype), stream, warmup, reps, ms_out);
+  return ms_time_ls_ex(A, lda, W_slices, ldw, S, m, n_slice, k, (void *const *)Y_chunks, ldy, in_dtype, MS_DTYPE_F32, stream, warmup, reps, ms_out);
 }
 
 MS_API int ms_time_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
                       float *const *Y_chunks, int ldy, int in_dtype, void *stream, int warmup, int reps, float *ms_out) {
-  const void *w1[1] = {W};
-  return timed(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, (void *const *)Y_chunks, ldy, in_dtype), stream, warmup, reps, ms_out);
+  return ms_time_rs_ex(X_slices, ldx, W, ldw, S, m_slice, n, k, (void *const *)Y_chunks, ldy, in_dtype, MS_DTYPE_F32, stream, warmup, reps, ms_out);
 }

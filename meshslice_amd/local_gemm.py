@@ -45,6 +45,69 @@ def _same(ts: Sequence[torch.Tensor], name: str):
     return s0
 
 
+class _Call:
+    """One validated local contraction: the C entry points' argument list up to (not including) ``stream``,
+    the device it runs on, the output it writes and the Python objects that keep the pointer tables alive."""
+
+    def __init__(self, device, args, out, keep):
+        self.device, self.args, self.out, self.keep = device, args, out, keep
+
+
+def _prepare_os(A_slices, B_slices, out, out_dtype) -> _Call:
+    a0 = _same(A_slices, "A_slices"); b0 = _same(B_slices, "B_slices")
+    if len(A_slices) != len(B_slices):
+        raise ValueError("A_slices and B_slices differ in length")
+    if a0.shape[1] != b0.shape[0] or a0.dtype != b0.dtype or a0.device != b0.device:
+        raise ValueError(f"slice shapes do not contract: {tuple(a0.shape)} @ {tuple(b0.shape)}")
+    m, k = a0.shape; n = b0.shape[1]
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype or a0.dtype, device=a0.device)
+    _check2d(out, "out")
+    if tuple(out.shape) != (m, n) or out.device != a0.device:
+        raise ValueError("out has the wrong shape or device")
+    pa, _ka = _lib.ptr_array([t.data_ptr() for t in A_slices])
+    pb, _kb = _lib.ptr_array([t.data_ptr() for t in B_slices])
+    args = (pa, pb, len(A_slices), m, n, k, a0.stride(0), b0.stride(0),
+            ctypes.c_void_p(out.data_ptr()), out.stride(0), _dt(a0), _dt(out))
+    return _Call(a0.device, args, out, (_ka, _kb))
+
+
+def _prepare_ls(A, W_slices, out, out_dtype) -> _Call:
+    _check2d(A, "A"); w0 = _same(W_slices, "W_slices")
+    if A.shape[1] != w0.shape[1] or A.dtype != w0.dtype or A.device != w0.device:
+        raise ValueError(f"shapes do not contract: {tuple(A.shape)} @ {tuple(w0.shape)}^T")
+    m, k = A.shape; ns = w0.shape[0]; S = len(W_slices)
+    dt = _chunk_dtype(out, out_dtype)
+    if out is None:
+        buf = torch.empty((S, m, ns), dtype=dt, device=A.device)
+        out = [buf[s] for s in range(S)]
+    o0 = _same(out, "out")
+    if len(out) != S or tuple(o0.shape) != (m, ns) or o0.dtype not in (torch.float32, torch.bfloat16) or o0.device != A.device:
+        raise ValueError("out must be S fp32 or bf16 chunks of shape [m, n_slice] on the operands' device")
+    pw, _kw = _lib.ptr_array([t.data_ptr() for t in W_slices])
+    py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
+    args = (ctypes.c_void_p(A.data_ptr()), A.stride(0), pw, w0.stride(0), S, m, ns, k, py, o0.stride(0), _dt(A), _dt(o0))
+    return _Call(A.device, args, list(out), (_kw, _ky))
+
+
+def _prepare_rs(X_slices, W, out, out_dtype) -> _Call:
+    _check2d(W, "W"); x0 = _same(X_slices, "X_slices")
+    if x0.shape[0] != W.shape[0] or x0.dtype != W.dtype or x0.device != W.device:
+        raise ValueError(f"shapes do not contract: {tuple(x0.shape)}^T @ {tuple(W.shape)}")
+    k, ms = x0.shape; n = W.shape[1]; S = len(X_slices)
+    dt = _chunk_dtype(out, out_dtype)
+    if out is None:
+        buf = torch.empty((S, ms, n), dtype=dt, device=W.device)
+        out = [buf[s] for s in range(S)]
+    o0 = _same(out, "out")
+    if len(out) != S or tuple(o0.shape) != (ms, n) or o0.dtype not in (torch.float32, torch.bfloat16) or o0.device != W.device:
+        raise ValueError("out must be S fp32 or bf16 chunks of shape [m_slice, n] on the operands' device")
+    px, _kx = _lib.ptr_array([t.data_ptr() for t in X_slices])
+    py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
+    args = (px, x0.stride(0), ctypes.c_void_p(W.data_ptr()), W.stride(0), S, ms, n, k, py, o0.stride(0), _dt(W), _dt(o0))
+    return _Call(W.device, args, list(out), (_kx, _ky))
+
+
 def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
             out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
             activation: Optional[str] = None, residual: Optional[torch.Tensor] = None,
@@ -54,24 +117,13 @@ def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
     Optional fused epilogue (bf16 operands): ``C = act(sum) + residual`` with ``activation='gelu'`` (tanh
     form) and ``residual`` of C's shape and dtype; ``row_moments=(row_sum, row_sumsq)`` are fp32 vectors of
     length m (either may be None) to which the row sums / sums of squares of the fp32 result are ADDED."""
-    a0 = _same(A_slices, "A_slices"); b0 = _same(B_slices, "B_slices")
-    if len(A_slices) != len(B_slices):
-        raise ValueError("A_slices and B_slices differ in length")
-    if a0.shape[1] != b0.shape[0] or a0.dtype != b0.dtype:
-        raise ValueError(f"slice shapes do not contract: {tuple(a0.shape)} @ {tuple(b0.shape)}")
-    m, k = a0.shape; n = b0.shape[1]
-    if out is None:
-        out = torch.empty((m, n), dtype=out_dtype or a0.dtype, device=a0.device)
-    _check2d(out, "out")
-    if tuple(out.shape) != (m, n):
-        raise ValueError("out has the wrong shape")
-    pa, _ka = _lib.ptr_array([t.data_ptr() for t in A_slices])
-    pb, _kb = _lib.ptr_array([t.data_ptr() for t in B_slices])
+    call = _prepare_os(A_slices, B_slices, out, out_dtype)
+    out = call.out
+    m, n = out.shape
     fused = activation is not None or residual is not None or row_moments is not None
     if not fused:
-        with torch.cuda.device(a0.device):
-            rc = _lib.load().ms_gemm_os(pa, pb, len(A_slices), m, n, k, a0.stride(0), b0.stride(0),
-                                        ctypes.c_void_p(out.data_ptr()), out.stride(0), _dt(a0), _dt(out), _stream())
+        with torch.cuda.device(call.device):
+            rc = _lib.load().ms_gemm_os(*call.args, _stream())
         _lib.check(rc)
         return out
     if activation not in (None, "gelu"):
@@ -79,18 +131,18 @@ def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
     res_ptr, ldr = None, 0
     if residual is not None:
         _check2d(residual, "residual")
-        if tuple(residual.shape) != (m, n) or residual.dtype != out.dtype:
-            raise ValueError("residual must have the shape and dtype of the output")
+        if tuple(residual.shape) != (m, n) or residual.dtype != out.dtype or residual.device != out.device:
+            raise ValueError("residual must have the shape, dtype and device of the output")
         res_ptr, ldr = ctypes.c_void_p(residual.data_ptr()), residual.stride(0)
     moments = [None, None]
     for idx, t in enumerate(row_moments or (None, None)):
         if t is not None:
-            if not (t.is_cuda and t.dtype == torch.float32 and t.dim() == 1 and t.numel() == m and t.is_contiguous()):
-                raise ValueError("row moments must be contiguous fp32 GPU vectors of length m")
+            if not (t.is_cuda and t.dtype == torch.float32 and t.dim() == 1 and t.numel() == m and t.is_contiguous()
+                    and t.device == out.device):
+                raise ValueError("row moments must be contiguous fp32 GPU vectors of length m on the output's device")
             moments[idx] = ctypes.c_void_p(t.data_ptr())
-    with torch.cuda.device(a0.device):
-        rc = _lib.load().ms_gemm_os_fused(pa, pb, len(A_slices), m, n, k, a0.stride(0), b0.stride(0),
-                                          ctypes.c_void_p(out.data_ptr()), out.stride(0), _dt(a0), _dt(out),
+    with torch.cuda.device(call.device):
+        rc = _lib.load().ms_gemm_os_fused(*call.args,
                                           _lib.MS_ACT_GELU if activation == "gelu" else _lib.MS_ACT_NONE,
                                           res_ptr, ldr, moments[0], moments[1], _stream())
     _lib.check(rc)
@@ -114,98 +166,77 @@ def gemm_ls(A: torch.Tensor, W_slices: Sequence[torch.Tensor],
     """``Y_s = A @ W_s^T``, W_s stored ``[n_slice, k]``.  Chunks are fp32 by default (exact partial sums for
     the reduce-scatter); ``out_dtype=torch.bfloat16`` gives what the reference's einsum returns for bf16
     operands (TensorParallel.py:181-189): one rounding of the fp32 accumulator, half the bytes."""
-    _check2d(A, "A"); w0 = _same(W_slices, "W_slices")
-    if A.shape[1] != w0.shape[1] or A.dtype != w0.dtype:
-        raise ValueError(f"shapes do not contract: {tuple(A.shape)} @ {tuple(w0.shape)}^T")
-    m, k = A.shape; ns = w0.shape[0]; S = len(W_slices)
-    dt = _chunk_dtype(out, out_dtype)
-    if out is None:
-        buf = torch.empty((S, m, ns), dtype=dt, device=A.device)
-        out = [buf[s] for s in range(S)]
-    o0 = _same(out, "out")
-    if len(out) != S or tuple(o0.shape) != (m, ns) or o0.dtype not in (torch.float32, torch.bfloat16):
-        raise ValueError("out must be S fp32 or bf16 chunks of shape [m, n_slice]")
-    pw, _kw = _lib.ptr_array([t.data_ptr() for t in W_slices])
-    py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
-    with torch.cuda.device(A.device):
-        rc = _lib.load().ms_gemm_ls_ex(ctypes.c_void_p(A.data_ptr()), A.stride(0), pw, w0.stride(0), S, m, ns, k,
-                                       py, o0.stride(0), _dt(A), _dt(o0), _stream())
+    call = _prepare_ls(A, W_slices, out, out_dtype)
+    with torch.cuda.device(call.device):
+        rc = _lib.load().ms_gemm_ls_ex(*call.args, _stream())
     _lib.check(rc)
-    return list(out)
+    return call.out
 
 
 def gemm_rs(X_slices: Sequence[torch.Tensor], W: torch.Tensor,
             out: Optional[List[torch.Tensor]] = None, out_dtype: Optional[torch.dtype] = None) -> List[torch.Tensor]:
     """``Y_s = X_s^T @ W``, X_s stored ``[k, m_slice]``; chunks fp32 by default, bf16 on request (see gemm_ls)."""
-    _check2d(W, "W"); x0 = _same(X_slices, "X_slices")
-    if x0.shape[0] != W.shape[0] or x0.dtype != W.dtype:
-        raise ValueError(f"shapes do not contract: {tuple(x0.shape)}^T @ {tuple(W.shape)}")
-    k, ms = x0.shape; n = W.shape[1]; S = len(X_slices)
-    dt = _chunk_dtype(out, out_dtype)
-    if out is None:
-        buf = torch.empty((S, ms, n), dtype=dt, device=W.device)
-        out = [buf[s] for s in range(S)]
-    o0 = _same(out, "out")
-    if len(out) != S or tuple(o0.shape) != (ms, n) or o0.dtype not in (torch.float32, torch.bfloat16):
-        raise ValueError("out must be S fp32 or bf16 chunks of shape [m_slice, n]")
-    px, _kx = _lib.ptr_array([t.data_ptr() for t in X_slices])
-    py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
-    with torch.cuda.device(W.device):
-        rc = _lib.load().ms_gemm_rs_ex(px, x0.stride(0), ctypes.c_void_p(W.data_ptr()), W.stride(0), S, ms, n, k,
-                                       py, o0.stride(0), _dt(W), _dt(o0), _stream())
+    call = _prepare_rs(X_slices, W, out, out_dtype)
+    with torch.cuda.device(call.device):
+        rc = _lib.load().ms_gemm_rs_ex(*call.args, _stream())
     _lib.check(rc)
-    return list(out)
+    return call.out
 
 
 def time_call(flow: str, operands, out, warmup: int = 5, reps: int = 20) -> List[float]:
     """Per-launch milliseconds (HIP events on the current stream) of one local contraction.
 
-    ``flow`` is 'os', 'ls' or 'rs'; ``operands``/``out`` are what gemm_os/gemm_ls/gemm_rs take."""
-    ms = (ctypes.c_float * reps)()
+    ``flow`` is 'os', 'ls' or 'rs'; ``operands`` / ``out`` are what gemm_os / gemm_ls / gemm_rs take (``out`` is
+    required here) and are checked the same way; LS / RS chunks may be fp32 or bf16."""
+    if flow not in ("os", "ls", "rs"):
+        raise ValueError(f"unknown dataflow {flow!r}")
+    if out is None:
+        raise ValueError("time_call needs the output buffer(s)")
+    if int(warmup) < 0 or int(reps) < 1:
+        raise ValueError("time_call needs warmup >= 0 and reps >= 1")
+    first, second = operands
     lib = _lib.load()
     if flow == "os":
-        A, B = operands
-        pa, _ka = _lib.ptr_array([t.data_ptr() for t in A]); pb, _kb = _lib.ptr_array([t.data_ptr() for t in B])
-        m, k = A[0].shape; n = B[0].shape[1]
-        rc = lib.ms_time_os(pa, pb, len(A), m, n, k, A[0].stride(0), B[0].stride(0), ctypes.c_void_p(out.data_ptr()),
-                            out.stride(0), _dt(A[0]), _dt(out), _stream(), warmup, reps, ms)
+        call, fn = _prepare_os(first, second, out, None), lib.ms_time_os
     elif flow == "ls":
-        A, W = operands
-        pw, _kw = _lib.ptr_array([t.data_ptr() for t in W]); py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
-        m, k = A.shape; ns = W[0].shape[0]
-        rc = lib.ms_time_ls(ctypes.c_void_p(A.data_ptr()), A.stride(0), pw, W[0].stride(0), len(W), m, ns, k,
-                            py, out[0].stride(0), _dt(A), _stream(), warmup, reps, ms)
-    elif flow == "rs":
-        X, W = operands
-        px, _kx = _lib.ptr_array([t.data_ptr() for t in X]); py, _ky = _lib.ptr_array([t.data_ptr() for t in out])
-        k, msl = X[0].shape; n = W.shape[1]
-        rc = lib.ms_time_rs(px, X[0].stride(0), ctypes.c_void_p(W.data_ptr()), W.stride(0), len(X), msl, n, k,
-                            py, out[0].stride(0), _dt(W), _stream(), warmup, reps, ms)
+        call, fn = _prepare_ls(first, second, out, None), lib.ms_time_ls_ex
     else:
-        raise ValueError(f"unknown dataflow {flow!r}")
+        call, fn = _prepare_rs(first, second, out, None), lib.ms_time_rs_ex
+    ms = (ctypes.c_float * int(reps))()
+    with torch.cuda.device(call.device):
+        rc = fn(*call.args, _stream(), int(warmup), int(reps), ms)
     _lib.check(rc)
     return list(ms)
 
 
-def mfma_stream_rate(operands: Optional[torch.Tensor] = None, iters: int = 4000, warmup: int = 20, reps: int = 200) -> float:
-    """FLOP/s that the current GPU sustains on a bare stream of the bf16 MFMA instruction the kernels are
-    built on (``ms_probe_mfma_stream``): the practical ceiling, under the device's power limit, for the
-    operand data given (default: N(0,1) values rounded to bf16, seed 0).  ``warmup + reps`` launches of about
-    a millisecond each, so the figure is the sustained one."""
+def mfma_stream_rate(operands: Optional[torch.Tensor] = None, iters: int = 4000, warmup: int = 20, reps: int = 200,
+                     shape: str = "32x32x16", waves_per_simd: int = 1) -> float:
+    """FLOP/s that the current GPU sustains on a bare stream of one bf16 MFMA instruction
+    (``ms_probe_mfma_stream_ex``): the practical ceiling, under the device's power limit, for the operand data
+    given (default: N(0,1) values rounded to bf16, seed 0).  ``shape`` is '32x32x16' (the instruction of the
+    big-tile kernels) or '16x16x32'; ``waves_per_simd`` 1 or 2.  ``warmup + reps`` launches of about a
+    millisecond each, so the figure is the sustained one."""
+    shapes = {"32x32x16": _lib.MS_MFMA_32X32X16, "16x16x32": _lib.MS_MFMA_16X16X32}
+    if shape not in shapes:
+        raise ValueError(f"unknown MFMA shape {shape!r} (one of {sorted(shapes)})")
+    if waves_per_simd not in (1, 2):
+        raise ValueError("waves_per_simd must be 1 or 2")
     dev = torch.device("cuda", torch.cuda.current_device())
+    need = 16 * 64 * 8
     if operands is None:
         g = torch.Generator(device="cpu").manual_seed(0)
-        operands = torch.randn(8 * 64 * 8, generator=g).to(torch.bfloat16).to(dev)
-    if not (operands.is_cuda and operands.dtype == torch.bfloat16 and operands.is_contiguous() and operands.numel() >= 8 * 64 * 8):
-        raise ValueError("operands must be a contiguous bf16 GPU tensor of at least 4096 elements")
+        operands = torch.randn(need, generator=g).to(torch.bfloat16).to(dev)
+    if not (operands.is_cuda and operands.dtype == torch.bfloat16 and operands.is_contiguous() and operands.numel() >= need):
+        raise ValueError(f"operands must be a contiguous bf16 GPU tensor of at least {need} elements")
     with torch.cuda.device(operands.device):
         cus = _lib.load().ms_query(_lib.MS_QUERY_CU_COUNT)
     if cus <= 0:
         raise _lib.MeshSliceError("could not read the compute-unit count of the device")
-    sink = torch.empty(256 * int(cus), dtype=torch.float32, device=operands.device)
+    sink = torch.empty(256 * waves_per_simd * int(cus), dtype=torch.float32, device=operands.device)
     ms, fl = ctypes.c_float(0.0), ctypes.c_double(0.0)
     with torch.cuda.device(operands.device):
-        rc = _lib.load().ms_probe_mfma_stream(ctypes.c_void_p(operands.data_ptr()), ctypes.c_void_p(sink.data_ptr()),
-                                              int(iters), int(warmup), int(reps), ctypes.byref(ms), ctypes.byref(fl), _stream())
+        rc = _lib.load().ms_probe_mfma_stream_ex(ctypes.c_void_p(operands.data_ptr()), ctypes.c_void_p(sink.data_ptr()),
+                                                 shapes[shape], int(waves_per_simd), int(iters), int(warmup), int(reps),
+                                                 ctypes.byref(ms), ctypes.byref(fl), _stream())
     _lib.check(rc)
     return fl.value / (ms.value * 1e-3)

@@ -497,16 +497,60 @@ def test_fused_epilogue_rejections():
         ms.gemm_os([h], [h], row_moments=(torch.zeros(63, device="cuda"), None))
 
 
-def test_mfma_stream_probe_reports_a_plausible_rate():
-    """The measurement aid runs, stays under the data-sheet peak and above a tenth of it, and rejects bad arguments."""
+@pytest.mark.parametrize("shape,wps", [("32x32x16", 1), ("32x32x16", 2), ("16x16x32", 1), ("16x16x32", 2)])
+def test_mfma_stream_probe_reports_a_plausible_rate(shape, wps):
+    """The measurement aid runs for either instruction shape at one and two waves per SIMD, stays under the
+    data-sheet peak and above a tenth of it."""
     from meshslice_amd.local_gemm import mfma_stream_rate
-    rate = mfma_stream_rate(iters=500, warmup=2, reps=5)
+    rate = mfma_stream_rate(iters=500, warmup=2, reps=5, shape=shape, waves_per_simd=wps)
     assert 0.25e15 < rate < 2.5166e15 * 1.02
+
+
+def test_mfma_stream_probe_rejects_bad_arguments():
+    from meshslice_amd.local_gemm import mfma_stream_rate
     L = _lib.load()
     ms_out, fl = ctypes.c_float(), ctypes.c_double()
-    x = torch.zeros(4096, dtype=torch.bfloat16, device="cuda"); sink = torch.zeros(256 * 256, device="cuda")
-    assert L.ms_probe_mfma_stream(None, ctypes.c_void_p(sink.data_ptr()), 10, 0, 1, ctypes.byref(ms_out), ctypes.byref(fl), None) == _lib.MS_ERR_ARG
-    assert L.ms_probe_mfma_stream(ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(sink.data_ptr()), 0, 0, 1, ctypes.byref(ms_out), ctypes.byref(fl), None) == _lib.MS_ERR_ARG
+    x = torch.zeros(8192, dtype=torch.bfloat16, device="cuda"); sink = torch.zeros(512 * 256, device="cuda")
+    xp, sp = ctypes.c_void_p(x.data_ptr()), ctypes.c_void_p(sink.data_ptr())
+    out = (ctypes.byref(ms_out), ctypes.byref(fl), None)
+    assert L.ms_probe_mfma_stream(None, sp, 10, 0, 1, *out) == _lib.MS_ERR_ARG
+    assert L.ms_probe_mfma_stream(xp, sp, 0, 0, 1, *out) == _lib.MS_ERR_ARG
+    assert L.ms_probe_mfma_stream_ex(xp, sp, 2, 1, 10, 0, 1, *out) == _lib.MS_ERR_ARG        # unknown shape
+    assert L.ms_probe_mfma_stream_ex(xp, sp, 0, 3, 10, 0, 1, *out) == _lib.MS_ERR_ARG        # three waves per SIMD
     with pytest.raises(ValueError):
         mfma_stream_rate(torch.zeros(16, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        mfma_stream_rate(shape="4x4x4")
 
+
+def test_time_call_checks_its_arguments_like_the_gemm_calls():
+    """The timing helper validates shapes, dtypes and devices before any pointer reaches the library, accepts bf16
+    chunks, and returns one positive time per repetition."""
+    A = torch.zeros((64, 32), dtype=torch.bfloat16, device="cuda"); B = torch.zeros((32, 48), dtype=torch.bfloat16, device="cuda")
+    W = torch.zeros((48, 32), dtype=torch.bfloat16, device="cuda"); Xt = torch.zeros((32, 64), dtype=torch.bfloat16, device="cuda")
+    C = torch.empty((64, 48), dtype=torch.bfloat16, device="cuda")
+    t = ms.time_call("os", ([A], [B]), C, warmup=1, reps=3)
+    assert len(t) == 3 and all(x > 0 for x in t)
+    for dt in (torch.float32, torch.bfloat16):
+        Y = [torch.empty((64, 48), dtype=dt, device="cuda")]
+        assert len(ms.time_call("ls", (A, [W]), Y, warmup=0, reps=2)) == 2
+        assert len(ms.time_call("rs", ([Xt], B), Y, warmup=0, reps=2)) == 2
+    small = [torch.empty((64, 40), dtype=torch.float32, device="cuda")]
+    with pytest.raises(ValueError):
+        ms.time_call("ls", (A, [W]), small)                      # undersized chunk
+    with pytest.raises(ValueError):
+        ms.time_call("rs", ([Xt], B), small)
+    with pytest.raises(ValueError):
+        ms.time_call("os", ([A], [B]), torch.empty((64, 40), dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        ms.time_call("os", ([A], [B.t()]), C)                    # not row-major
+    with pytest.raises(ValueError):
+        ms.time_call("ls", (A, [W]), [torch.empty((64, 48), dtype=torch.float16, device="cuda")])
+    with pytest.raises(ValueError):
+        ms.time_call("os", ([A], [B]), None)
+    with pytest.raises(ValueError):
+        ms.time_call("xs", ([A], [B]), C)
+    with pytest.raises(ValueError):
+        ms.time_call("os", ([A], [B]), C, reps=0)
+    with pytest.raises(_lib.MeshSliceError):
+        ms.time_call("os", ([A.cpu()], [B.cpu()]), C)

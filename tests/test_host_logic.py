@@ -249,3 +249,65 @@ def test_shipped_compute_term_loads_and_feeds_the_models():
         assert steady >= 4 * t
     finally:
         CostModel.use_compute_term(None)
+
+
+def test_autotuner_class_mirrors_the_reference_surface():
+    """``Autotuner(graph, shapes).emulateFFTime(meshshape, sweep)`` -> (seconds, {node name: slice count}), the
+    dataflow rule and the transposition flip of 'rs' layers (reference Autotuner.py:278-313, :391-426)."""
+    class Flat(CostModel.ComputeTerm):
+        def seconds(self, M, N, K, layout):
+            return 2.0 * M * N * K / 1.5e15 + 5e-6
+    layers = [("in_proj", 16384, 12288, 36864), ("out_proj", 16384, 12288, 12288),
+              ("ff1", 16384, 12288, 49152), ("ff2", 16384, 49152, 12288)]
+    graph = Autotuner.LayerGraph(layers)
+    assert graph.nodenames[:2] == ["Input:in_proj", "in_proj"] and graph.nodes["ff1"]["op_type"] == "FeedForward"
+    shapes = [(2, 8), (4, 4), (8, 2)]
+    CostModel.use_compute_term(Flat())
+    try:
+        tuner = Autotuner.Autotuner(graph, shapes, bestshape=(4, 4))
+        assert tuner.dataflows == {"in_proj": "os", "out_proj": "ls", "ff1": "os", "ff2": "ls"}
+        assert not any(tuner.transposition.values())
+        total, ks = tuner.emulateFFTime((4, 4), sweep=True)
+        flat_total, flat_best = Autotuner.emulateFFTime([(B, I, O, tuner.dataflows[n]) for n, B, I, O in layers], (4, 4), sweep=True)
+        assert list(ks) == [n for n, *_ in layers] and list(ks.values()) == flat_best
+        # the class prices the mesh with the reference's 242 * 1024**4 FLOP/s figure, the free function with the MI355X peak;
+        # neither enters the model times, which come from the installed compute term
+        assert total == pytest.approx(flat_total, rel=1e-12)
+        # neighbour search: ends on a shape that none of its neighbours beats, and sweep finds the global best
+        best, ksplits = tuner.emulatedFinetune()
+        times = {s: tuner.emulateFFTime(s)[0] for s in shapes}
+        i = shapes.index(best)
+        assert all(times[best] <= times[shapes[j]] for j in (i - 1, i + 1) if 0 <= j < len(shapes))
+        assert ksplits == tuner.emulateFFTime(best)[1]
+        tuner2 = Autotuner.Autotuner(graph, shapes)
+        assert tuner2.bestshape == (2, 8)
+        best2, _ = tuner2.emulatedFinetune(sweep=True)
+        swept = {s: tuner2.emulateFFTime(s, sweep=True)[0] for s in shapes}
+        assert swept[best2] == min(swept.values())
+    finally:
+        CostModel.use_compute_term(None)
+    # an 'rs' layer (weight largest) flips the transposition of what follows it
+    chain = Autotuner.LayerGraph([("small", 64, 4096, 4096)])
+    chain.nodenames.append("next")
+    chain.nodes["next"] = {"op_name": "next", "op_type": "Gelu", "inputs": ("small",), "shape": [64, 4096]}
+    t = Autotuner.Autotuner(chain, [(2, 2)])
+    assert t.dataflows["small"] == "rs" and t.transposition == {"Input:small": False, "small": True, "next": True}
+    with pytest.raises(ValueError):
+        Autotuner.Autotuner(graph, shapes, bestshape=(3, 3))
+
+
+def test_both_shipped_compute_terms_load_and_the_ones_term_is_the_faster():
+    """The default term is fitted on N(0, 0.02) operands; the reference's all-ones protocol stays selectable and, on
+    this power-limited device, reads faster for every layout."""
+    try:
+        normal = CostModel.load_compute_term()
+        ones = CostModel.load_compute_term(operands="ones")
+        assert set(normal.eta) == set(ones.eta) == {"nn", "nt", "tn"}
+        for lay in normal.eta:
+            assert 0.2 < normal.eta[lay] < ones.eta[lay] < 1.0
+        with pytest.raises(ValueError):
+            CostModel.load_compute_term(operands="zeros")
+        with pytest.raises(ValueError):
+            CostModel.estimateMatmul(None, 8, 8, 8, operands="zeros")
+    finally:
+        CostModel.use_compute_term(None)
