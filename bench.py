@@ -22,10 +22,14 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6     # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
-# Bytes per launch of the config-2 kernel that cross the L2 <-> fabric boundary (Infinity Cache or HBM), from
-# two rocprofv3 --pmc runs (FETCH_SIZE 692250 KiB-units x 2.0 and WRITE_SIZE 104960 x 1.0, each scaled by what
-# the same counter reads for a 1 GiB device copy in the same run); summary in profiles/gemm_bf16_big_256x384x64_os_cfg2.md.
-MEASURED_TRAFFIC_BYTES = 1525127376
+PEAK_FP32_TFLOPS = 157.3      # MI355X dense fp32 MFMA
+# Bytes per launch of the config-2 kernel that cross the L2 <-> fabric boundary (Infinity Cache or HBM).  This is an
+# OFFLINE figure: two rocprofv3 --pmc runs of this program (FETCH_SIZE 692250 KiB-units x 2.0 and WRITE_SIZE 104960 x 1.0,
+# each scaled by what the same counter reads for a 1 GiB device copy in the same run), valid for the kernel variant
+# named beside it.  It is reported only when the launch this run timed used that variant (ms_query tells).
+TRAFFIC_PROFILE = {"bytes": 1525127376, "variant": 10,
+                   "source": "profiles/gemm_bf16_big_256x384x64_os_cfg2.md @ variant 10 (gemm_bf16_big_kernel<4,6>, 256x384x64 tile)"}
+SETTLE_LAUNCHES = 60          # untimed launches before the warm-up: the package power controller's start-up transient
 
 
 def sel_index(L, S, B, k):
@@ -127,26 +131,43 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # ---- timed region: W warm-up steps, then exactly K steps between two synchronisations
-    for _ in range(args.warmup):
+    # ---- settle phase (always, whatever --warmup says): the first launches after an idle period run up to 30 % slow
+    for _ in range(SETTLE_LAUNCHES):
         ms.gemm_os(A, B, out=C)
     torch.cuda.synchronize()
+    variant = int(lib.ms_query(_lib.MS_QUERY_LAST_VARIANT))
+    launches = int(lib.ms_query(_lib.MS_QUERY_LAST_LAUNCHES))
+
+    # ---- timed region: W warm-up steps, then exactly K steps between two synchronisations; two HIP events on the
+    # launch stream bracket the same K launches, so their mean is the kernel's duration in THIS region
+    for _ in range(args.warmup):
+        ms.gemm_os(A, B, out=C)
+    e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
+    e0.record()
     for _ in range(args.steps):
         ms.gemm_os(A, B, out=C)
+    e1.record()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     value = flops / (ms_per_step * 1e-3) / 1e12
+    k_ms = e0.elapsed_time(e1) / args.steps
 
-    # ---- kernel duration with HIP events around every launch, on the launch stream
-    # (the package power controller needs some tens of launches to settle: short runs read ~8 % slower)
+    # the same launches bracketed one by one (each followed by a host wait, which lets the device idle between
+    # launches: these read a little differently from back-to-back launches and are reported for information)
     per_launch = ms.time_call("os", (A, B), C, warmup=2, reps=min(max(args.steps, 10), 100))
-    k_ms = float(np.mean(per_launch))
     achieved = flops / (k_ms * 1e-3) / 1e12
+    traffic_ok = variant == TRAFFIC_PROFILE["variant"] and launches == 1
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                "kernel_ms_mean": round(k_ms, 4), "kernel_ms_median": round(median(per_launch), 4),
-                "kernel_ms_min": round(float(np.min(per_launch)), 4),
+                "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                "traffic": TRAFFIC_PROFILE["bytes"] if traffic_ok else None,
+                "traffic_source": TRAFFIC_PROFILE["source"] if traffic_ok else
+                f"none: this run launched variant {variant} ({launches} launch(es)), the profile covers variant {TRAFFIC_PROFILE['variant']}",
+                "kernel_variant": variant,
+                "kernel_ms_mean": round(k_ms, 4), "kernel_ms_how": f"two HIP events on the launch stream around the {args.steps} timed launches",
+                "kernel_ms_single_launch_mean": round(float(np.mean(per_launch)), 4),
+                "kernel_ms_single_launch_min": round(float(np.min(per_launch)), 4),
                 "algorithmic_flops_per_launch": flops,
                 "algorithmic_hbm_bytes_per_launch": 2 * (M * K + K * N + M * N)}
 
@@ -156,20 +177,43 @@ def main():
     want = X[rows].float().cpu().numpy().astype(np.float64) @ W.float().cpu().numpy().astype(np.float64)
     extra["parity_rel_frobenius_sampled_rows"] = float(f"{orc.rel_frobenius(C[rows].float().cpu().numpy(), want):.3e}")
 
+    def _sustained(f, n, warm=10):
+        """mean ms per launch of n back-to-back launches between two HIP events on the launch stream"""
+        for _ in range(warm):
+            f()
+        a = torch.cuda.Event(enable_timing=True); b = torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            f()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n
+
+    out_extra = {}
     if not args.only_main:
+        n_side = min(max(args.steps, 20), 100)
+        # S = 1 against S = 4, measured the same way and interleaved (A B A B), best of each
         C1 = torch.empty_like(C)
-        t_s1 = median(ms.time_call("os", ([X], [W]), C1, warmup=3, reps=min(max(args.steps, 10), 50)))
-        t_s4 = median(per_launch)
+        t_s4, t_s1 = [], []
+        for _ in range(2):
+            t_s4.append(_sustained(lambda: ms.gemm_os(A, B, out=C), n_side))
+            t_s1.append(_sustained(lambda: ms.gemm_os([X], [W], out=C1), n_side))
+        t_s4, t_s1 = min(t_s4), min(t_s1)
         extra["os_s1_ms"] = round(t_s1, 4)
         extra["os_s4_ms"] = round(t_s4, 4)
+        extra["os_s1_tflops"] = round(flops / t_s1 / 1e9, 1)
         extra["slicing_overhead_s4_vs_s1"] = round(t_s4 / t_s1 - 1.0, 4)
         del C1
         # config 3: LS, S=8 -> 8 fp32 chunks [4096,1536]
         idx8 = [torch.from_numpy(sel_index(12288, 8, 8, k)).cuda() for k in range(8)]
         Ws = [W[i, :].contiguous() for i in idx8]
         Y = [torch.empty((4096, 1536), dtype=torch.float32, device="cuda") for _ in range(8)]
-        t = median(ms.time_call("ls", (X, Ws), Y, warmup=3, reps=min(max(args.steps, 10), 50)))
+        t = _sustained(lambda: ms.gemm_ls(X, Ws, out=Y), n_side)
         extra["ls_s8_ms"] = round(t, 4); extra["ls_s8_tflops"] = round(flops / t / 1e9, 1)
+        out_extra["roofline_ls"] = {"workload": "config 3: LS, A[4096,12288] x 8 slices W_s[1536,12288]^T -> 8 fp32 chunks", "bound": "mfma",
+                                    "achieved": round(flops / t / 1e9, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                    "frac": round(flops / t / 1e9 / PEAK_BF16_TFLOPS, 4), "kernel_ms_mean": round(t, 4),
+                                    "kernel_variant": int(lib.ms_query(_lib.MS_QUERY_LAST_VARIANT))}
         del Ws, Y
         # config 4: RS, S=4 -> 4 fp32 chunks [768,12288]
         g = torch.Generator(device="cuda").manual_seed(4)
@@ -178,9 +222,28 @@ def main():
         idx4 = [torch.from_numpy(sel_index(3072, 4, 8, k)).cuda() for k in range(4)]
         Xs = [X4[:, i].contiguous() for i in idx4]
         Y = [torch.empty((768, 12288), dtype=torch.float32, device="cuda") for _ in range(4)]
-        t = median(ms.time_call("rs", (Xs, dY), Y, warmup=3, reps=min(max(args.steps, 10), 50)))
-        extra["rs_s4_ms"] = round(t, 4); extra["rs_s4_tflops"] = round(2.0 * 3072 * 12288 * 4096 / t / 1e9, 1)
+        fl4 = 2.0 * 3072 * 12288 * 4096
+        t = _sustained(lambda: ms.gemm_rs(Xs, dY, out=Y), 2 * n_side)
+        extra["rs_s4_ms"] = round(t, 4); extra["rs_s4_tflops"] = round(fl4 / t / 1e9, 1)
+        out_extra["roofline_rs"] = {"workload": "config 4: RS, 4 slices X_s[4096,768]^T x dY[4096,12288] -> 4 fp32 chunks", "bound": "mfma",
+                                    "achieved": round(fl4 / t / 1e9, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                                    "frac": round(fl4 / t / 1e9 / PEAK_BF16_TFLOPS, 4), "kernel_ms_mean": round(t, 4),
+                                    "kernel_variant": int(lib.ms_query(_lib.MS_QUERY_LAST_VARIANT))}
         del Xs, Y, X4, dY
+        # the fp32 path against the fp32 MFMA peak: config 1 (device block 512x512x1024 in four K slices) and one 4096^3 product
+        g = torch.Generator(device="cuda").manual_seed(1)
+        A1 = [torch.randn((512, 256), generator=g, device="cuda") for _ in range(4)]
+        B1 = [torch.randn((256, 512), generator=g, device="cuda") for _ in range(4)]
+        C32 = torch.empty((512, 512), device="cuda")
+        t = _sustained(lambda: ms.gemm_os(A1, B1, out=C32), 200)
+        extra["fp32_config1_ms"] = round(t, 5); extra["fp32_config1_tflops"] = round(2.0 * 512 * 512 * 1024 / t / 1e9, 2)
+        A32 = torch.randn((4096, 4096), generator=g, device="cuda"); B32 = torch.randn((4096, 4096), generator=g, device="cuda")
+        C32 = torch.empty((4096, 4096), device="cuda")
+        t = _sustained(lambda: ms.gemm_os([A32], [B32], out=C32), 20, warm=3)
+        out_extra["roofline_fp32"] = {"workload": "fp32 4096 x 4096 x 4096, one slice", "bound": "mfma",
+                                      "achieved": round(2.0 * 4096 ** 3 / t / 1e9, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                                      "frac": round(2.0 * 4096 ** 3 / t / 1e9 / PEAK_FP32_TFLOPS, 4), "kernel_ms_mean": round(t, 4)}
+        del A1, B1, A32, B32, C32
         # fused epilogue: GELU folded into the config-2 product vs the product followed by a separate GELU kernel
         def _events(f, n):
             for _ in range(3):
@@ -232,8 +295,10 @@ def main():
                                "S=4 block-cyclic K slices of 3072, fp32 accumulate, C[4096,12288] bf16",
                    "S": S, "m": M, "n": N, "k_slice": K // S, "blocksize": 8},
         "pct_of_bf16_mfma_peak": round(100.0 * value / PEAK_BF16_TFLOPS, 2),
+        "settle_launches": SETTLE_LAUNCHES,
         "roofline": roofline,
     }
+    out.update(out_extra)
     if not args.no_cpu_baseline:
         A_host = [a.float().cpu().numpy() for a in A]
         B_host = [b.float().cpu().numpy() for b in B]

@@ -23,6 +23,8 @@
 #ifndef MESHSLICE_HIP_H
 #define MESHSLICE_HIP_H
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -45,6 +47,9 @@ extern "C" {
 #define MS_QUERY_MAX_SLICES 4   /* MS_MAX_SLICES */
 #define MS_QUERY_LAST_LAUNCHES 5 /* kernels launched by the calling thread's last ms_gemm_* call (a product whose tiles
                                    would leave much of the last round of compute units idle is done in two launches) */
+#define MS_QUERY_LAST_SPLITS 7   /* ways in which that launch split the contraction (1: not split) */
+#define MS_QUERY_LAST_VARIANT 6  /* bf16 kernel variant (tile shape, see ms_set_variant) of the first of those launches; 0 for
+                                   the fp32 kernel.  Lets a measurement name the kernel it timed. */
 
 /* Library version, major*10000 + minor*100 + patch. */
 int ms_version(void);
@@ -84,6 +89,33 @@ int ms_gemm_os_fused(const void *const *A_slices, const void *const *B_slices, i
                      void *C, int ldc, int in_dtype, int out_dtype,
                      int activation, const void *residual, int ldr,
                      float *row_sum, float *row_sumsq, void *stream);
+
+/* Output-stationary with a workspace: ms_gemm_os_fused (activation MS_ACT_NONE, residual / row_sum / row_sumsq NULL: the
+ * plain product of ms_gemm_os) that may split the contraction.  A product with a small output and a long contraction
+ * (the backward-data GEMM of an LHS-stationary layer on a large mesh: 2048 x 1536 x 12288 is 64 tiles for 256 compute
+ * units) leaves most of the device idle if every output tile is one work item.  With a workspace the call may cut the
+ * K range of every tile into 2..8 parts that run on different compute units; each part leaves its fp32 partial tile in
+ * the workspace, and the part that finishes last adds them up in a fixed order (so the result does not depend on
+ * timing: the same call gives the same bits every time) and writes its part of C.  Only the plain product is split: with
+ * an activation, a residual or row moments the call runs as ms_gemm_os_fused does.  No counterpart in the reference, where
+ * XLA picks the contraction's schedule.
+ * workspace: device memory, 256-byte aligned, prepared once with ms_workspace_init and then reusable by any number of
+ * calls, one at a time (calls that share a workspace must not overlap: same stream, or ordered by events);
+ * ms_workspace_bytes() is the size with which no product is refused a split for lack of room, a smaller one only
+ * narrows the choice.  workspace == NULL behaves like ms_gemm_os_fused. */
+int ms_gemm_os_ws(const void *const *A_slices, const void *const *B_slices, int S,
+                  int m, int n, int k_slice, int lda, int ldb,
+                  void *C, int ldc, int in_dtype, int out_dtype,
+                  int activation, const void *residual, int ldr,
+                  float *row_sum, float *row_sumsq,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/* Bytes of workspace that let every product split its contraction on the current device (0 on a HIP error). */
+size_t ms_workspace_bytes(void);
+
+/* Prepares a workspace for ms_gemm_os_ws: clears its arrival counters (the first 4096 bytes) on `stream`.  Needed once
+ * after allocation; every call leaves the counters cleared again. */
+int ms_workspace_init(void *workspace, size_t bytes, void *stream);
 
 /* LHS-stationary: for s < S, Y_s[m,n_slice] = A[m,k] @ W_s[n_slice,k]^T  (fp32 out).
  * Replaces the contractions of MeshFlow_LS (TensorParallel.py:181,187); S == 1 is Collective_LS
@@ -130,7 +162,12 @@ int ms_time_rs(const void *const *X_slices, int ldx, const void *W, int ldw, int
                int m_slice, int n, int k,
                float *const *Y_chunks, int ldy, int in_dtype, void *stream,
                int warmup, int reps, float *ms_out);
-/* The same for ms_gemm_ls_ex / ms_gemm_rs_ex (chunks in out_dtype). */
+/* The same for ms_gemm_os_ws (plain product) and for ms_gemm_ls_ex / ms_gemm_rs_ex (chunks in out_dtype). */
+int ms_time_os_ws(const void *const *A_slices, const void *const *B_slices, int S,
+                  int m, int n, int k_slice, int lda, int ldb,
+                  void *C, int ldc, int in_dtype, int out_dtype,
+                  void *workspace, size_t workspace_bytes, void *stream,
+                  int warmup, int reps, float *ms_out);
 int ms_time_ls_ex(const void *A, int lda, const void *const *W_slices, int ldw, int S,
                   int m, int n_slice, int k,
                   void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream,
@@ -189,8 +226,9 @@ int ms_probe_mfma_stream_ex(const void *operands, float *sink, int shape, int wa
 int ms_probe_mfma_stream(const void *operands, float *sink, int iters, int warmup, int reps,
                          float *ms_out, double *flops_per_launch, void *stream);
 
-/* Tuning knob for experiments: selects the bf16 kernel variant used by later calls on this
- * thread (0 = library default).  Unknown ids are rejected with MS_ERR_ARG. */
+/* Hook for tests and measurements (thread-local): later bf16 calls on this thread use tile variant `variant % 100`
+ * (1..11, 0 = the library's choice) and split the contraction `variant / 100` ways (2..8, 0 = the library's choice;
+ * a forced split needs a workspace and an output-stationary product).  Unknown ids are rejected with MS_ERR_ARG. */
 int ms_set_variant(int variant);
 
 #ifdef __cplusplus

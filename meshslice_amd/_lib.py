@@ -22,6 +22,8 @@ MS_QUERY_IS_GFX950 = 2
 MS_QUERY_LDS_BYTES = 3
 MS_QUERY_MAX_SLICES = 4
 MS_QUERY_LAST_LAUNCHES = 5
+MS_QUERY_LAST_VARIANT = 6
+MS_QUERY_LAST_SPLITS = 7
 MS_ACT_NONE = 0
 MS_ACT_GELU = 1
 MS_MFMA_32X32X16 = 0
@@ -32,7 +34,7 @@ LIB_PATH = os.path.join(_HERE, "libmeshslice_hip.so")
 
 EXPORTS = (
     "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
-    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex",
+    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_os_ws", "ms_workspace_bytes", "ms_workspace_init", "ms_time_os_ws", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex",
     "ms_time_os", "ms_time_ls", "ms_time_rs", "ms_time_ls_ex", "ms_time_rs_ex",
     "ms_pack_slices", "ms_unpack_chunks", "ms_probe_mfma_stream", "ms_probe_mfma_stream_ex",
 )
@@ -63,6 +65,15 @@ def _declare(lib):
     lib.ms_gemm_os_fused.argtypes = os_args[:-1] + [c_int, c_vp, c_int, c_vp, c_vp, c_vp]
     lib.ms_gemm_os_fused.restype = c_int
     lib.ms_gemm_os.argtypes = os_args
+    # ..., out_dtype, activation, residual, ldr, row_sum, row_sumsq, workspace, workspace_bytes, stream
+    lib.ms_gemm_os_ws.argtypes = os_args[:-1] + [c_int, c_vp, c_int, c_vp, c_vp, c_vp, ctypes.c_size_t, c_vp]
+    lib.ms_gemm_os_ws.restype = c_int
+    lib.ms_time_os_ws.argtypes = os_args[:-1] + [c_vp, ctypes.c_size_t, c_vp, c_int, c_int, fp]
+    lib.ms_time_os_ws.restype = c_int
+    lib.ms_workspace_bytes.argtypes = []
+    lib.ms_workspace_bytes.restype = ctypes.c_size_t
+    lib.ms_workspace_init.argtypes = [c_vp, ctypes.c_size_t, c_vp]
+    lib.ms_workspace_init.restype = c_int
     lib.ms_gemm_ls.argtypes = ls_args
     lib.ms_gemm_rs.argtypes = rs_args
     lib.ms_gemm_ls_ex.argtypes = ls_args[:-1] + [c_int, c_vp]      # ..., in_dtype, out_dtype, stream

@@ -5,6 +5,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "ms_common.hip.inc"
 
@@ -61,29 +62,38 @@ int msi::fail(int code, const char *fmt, ...) {
 namespace {
 
 thread_local int g_variant = 0;
+thread_local int g_splits = 0;    // forced split count of the contraction (0 = library default)
 thread_local int g_launches = 0;   // kernels launched by the last GEMM call of this thread
+thread_local int g_last_variant = 0;   // bf16 kernel variant of that call's first launch (0: the fp32 kernel)
+thread_local int g_last_splits = 1;    // and the number of ways it split the contraction
 
 using msi::fail;
 
 struct DevInfo {
-  int valid, cus, clock_khz, gfx950, lds;
+  std::once_flag once;
+  hipError_t err = hipSuccess;
+  int cus = 0, clock_khz = 0, gfx950 = 0, lds = 0;
 };
 DevInfo g_dev[64];
 
+// Facts about the calling thread's current device, read from the runtime once per ordinal (call_once: concurrent
+// first calls from several host threads wait for the one that fills the entry).
 int dev_info(DevInfo **out) {
   int d = 0;
   MS_HIP(hipGetDevice(&d));
   if (d < 0 || d >= 64) return fail(MS_ERR_HIP, "device ordinal %d out of range", d);
-  if (!__atomic_load_n(&g_dev[d].valid, __ATOMIC_ACQUIRE)) {
+  DevInfo &di = g_dev[d];
+  std::call_once(di.once, [&di, d]() {
     hipDeviceProp_t p;
-    MS_HIP(hipGetDeviceProperties(&p, d));
-    g_dev[d].cus = p.multiProcessorCount;
-    g_dev[d].clock_khz = p.clockRate;
-    g_dev[d].gfx950 = strncmp(p.gcnArchName, "gfx950", 6) == 0;
-    g_dev[d].lds = (int)p.sharedMemPerBlock;
-    __atomic_store_n(&g_dev[d].valid, 1, __ATOMIC_RELEASE);
-  }
-  *out = &g_dev[d];
+    di.err = hipGetDeviceProperties(&p, d);
+    if (di.err != hipSuccess) return;
+    di.cus = p.multiProcessorCount;
+    di.clock_khz = p.clockRate;
+    di.gfx950 = strncmp(p.gcnArchName, "gfx950", 6) == 0;
+    di.lds = (int)p.sharedMemPerBlock;
+  });
+  if (di.err != hipSuccess) return fail(MS_ERR_HIP, "hipGetDeviceProperties failed: %s", hipGetErrorString(di.err));
+  *out = &di;
   return MS_OK;
 }
 
@@ -106,7 +116,16 @@ struct Problem {
   int ldr = 0;
   float *row_sum = nullptr;
   float *row_sumsq = nullptr;
+  // workspace for split contractions (null / 0: none, the contraction is never split)
+  void *ws = nullptr;
+  size_t ws_bytes = 0;
 };
+
+// Layout of a split-contraction workspace: SPLIT_MAX_BANDS arrival counters per output tile, then one fp32 partial tile
+// per work item.
+constexpr size_t WS_HEADER_BYTES = 4096;
+constexpr int WS_COUNTERS = (int)(WS_HEADER_BYTES / sizeof(int));
+constexpr int WS_MAX_TILES = WS_COUNTERS / msk::SPLIT_MAX_BANDS;     // output tiles of a split product
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -139,6 +158,8 @@ int validate(const Problem &p) {
     if (!aligned16(p.res)) return fail(MS_ERR_ARG, "%s: residual pointer not 16-byte aligned", fn);
     if (p.ldr < p.N || p.ldr % qo) return fail(MS_ERR_ARG, "%s: residual leading dimension %d must be >= n and a multiple of %d", fn, p.ldr, qo);
   }
+  if (p.ws && ((reinterpret_cast<uintptr_t>(p.ws) & 255) || p.ws_bytes < WS_HEADER_BYTES))
+    return fail(MS_ERR_ARG, "%s: a workspace must be 256-byte aligned and hold at least %zu bytes", fn, WS_HEADER_BYTES);
   if ((reinterpret_cast<uintptr_t>(p.row_sum) | reinterpret_cast<uintptr_t>(p.row_sumsq)) & 3) return fail(MS_ERR_ARG, "%s: row-moment pointers must be 4-byte aligned", fn);
   if ((p.act || p.res || p.row_sum || p.row_sumsq) && (p.flow != OS || p.in_dtype != MS_DTYPE_BF16))
     return fail(MS_ERR_UNSUPPORTED, "%s: the fused epilogue exists for the output-stationary bf16 kernel only", fn);
@@ -159,9 +180,12 @@ void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
   }
 }
 
-// tile BM x BN, WGM x WGN waves, NS ring stages of BK_ k-elements
+extern const char *const SPLIT_REFUSALS[];
+int split_refused(const Problem &p, const DevInfo &dev, int variant, int splits);
+
+// tile BM x BN, WGM x WGN waves, NS ring stages of BK_ k-elements; contraction split `splits` ways
 template <int BM, int BN, int WGM, int WGN, int BK_, int NS, bool BIG = false>
-int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream, int variant, int splits) {
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
   for (int i = 0; i < p.na; i++) g.a[i] = p.a[i];
@@ -179,7 +203,16 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   if (total > 0x7FFFFFFF) return fail(MS_ERR_ARG, "problem has too many tiles");
   g.total_tiles = (int)total;
   g.group_m = 8;
-  int grid = dev.cus < g.total_tiles ? dev.cus : g.total_tiles;
+  g.splits = 1;
+  if (splits > 1) {
+    const int why = split_refused(p, dev, variant, splits);
+    if (why) return fail(MS_ERR_ARG, "contraction cannot be split %d ways here: %s", splits, SPLIT_REFUSALS[why]);
+    g.splits = splits;
+    g.ws_count = static_cast<int *>(p.ws);
+    g.ws_tiles = static_cast<char *>(p.ws) + WS_HEADER_BYTES;
+  }
+  const long items = total * g.splits;
+  int grid = dev.cus < items ? dev.cus : (int)items;
   dim3 gd(grid), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   g.act = p.act; g.res = p.res; g.ldr = p.ldr; g.row_sum = p.row_sum; g.row_sumsq = p.row_sumsq;
@@ -210,45 +243,91 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
 //   7: 256x256, 8 waves, 2 x 64     8: 256x192, 4 waves, 2 x 64     9: 192x256, 4 waves, 2 x 64
 //  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel<4, 6>)     11: 384x192, 4 waves, 2 x 64 (gemm_bf16_big_kernel<6, 3>)
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
-// ceil(tiles / CUs) rounds of one tile per CU, so the estimate is rounds x tile area / relative tile
+// ceil(work items / CUs) rounds of one item per CU, so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile reaches 1.06
 // with a k-contiguous A and 1.02 without, the 384x192 tile 1.04 and 0.96, 192-wide ring tiles about 0.93,
 // 128x128 tiles about 0.55).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
 // k-contiguous: whole 128-byte lines per request, half as many barriers as 32-deep stages.
-struct Pick { int v; double cost; };
+//
+// An output-stationary product with fewer tiles than compute units may split its contraction (work items = tiles x
+// splits, see split_k_exchange): a split item costs 1 / splits of the tile, and the whole launch pays for the exchange
+// of partial tiles, which is bound by memory bandwidth (splits x m x n fp32 values written through to memory and read
+// back: about 2.8 TB/s) plus a fixed few microseconds.  In the estimate's units (tile area x share of the contraction,
+// one compute unit doing about 5.7 TFLOP/s) that is (SPLIT_FIX + splits x m x n x SPLIT_PER_ELEMENT) / K.  Measured on
+// 2048 x 1536 x 12288 (64 tiles of 256x192): 170 us unsplit, 100 / 85 / 88 us with 2 / 3 / 4 splits.
+struct Pick { int v, splits; double cost; };
 
-// the single tile shape with the lowest estimated cost for the whole problem
+constexpr int VARIANTS = 11;
+struct TileShape { int bm, bn; };
+constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256}, {128, 128}, {256, 256}, {256, 192},
+                                             {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192}};
+constexpr int SPLIT_CHOICES[] = {1, 2, 3, 4, 6, 8};
+constexpr int SPLIT_MAX = 8;
+constexpr long SPLIT_MIN_K = 512;            // contraction elements per split item, at least
+constexpr double SPLIT_FIX = 1.4e7;          // fixed cost of an exchange (about 5 us)
+constexpr double SPLIT_PER_ELEMENT = 8.2;    // per split and output element (8 bytes through memory)
+
+const char *const SPLIT_REFUSALS[] = {"", "only output-stationary products split their contraction", "no workspace was given",
+                                      "more work items than compute units", "too many output tiles for the workspace's counters",
+                                      "the partial tiles do not fit the workspace", "too few contraction steps per split",
+                                      "split count outside [2, 8]", "this tile variant has no split path",
+                                      "products with a fused epilogue are not split"};
+
+// 0 if problem p can run on tile variant v with its contraction split `splits` ways, else an index into SPLIT_REFUSALS
+int split_refused(const Problem &p, const DevInfo &dev, int v, int splits) {
+  const int bm = TILE_OF[v].bm, bn = TILE_OF[v].bn;
+  if (splits < 2 || splits > SPLIT_MAX) return 7;
+  if (v == 1 || v == 4) return 8;     // 256x256 on four waves: see ring_can_split
+  if (p.act || p.res || p.row_sum || p.row_sumsq) return 9;   // see ring_can_split, big_can_split
+  if (p.flow != OS) return 1;
+  if (!p.ws) return 2;
+  const long tiles = (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
+  if (tiles * splits > dev.cus) return 3;
+  if (tiles > WS_MAX_TILES) return 4;
+  if ((size_t)(tiles * splits) * bm * bn * sizeof(float) + WS_HEADER_BYTES > p.ws_bytes) return 5;
+  if (((long)(p.K + 63) / 64) * p.S < splits) return 6;     // every part needs at least one 64-deep K step
+  return 0;
+}
+
+// the tile shape and split count with the lowest estimated cost for the whole problem
 Pick pick_variant(const Problem &p, const DevInfo &dev) {
-  struct Cand { int v, bm, bn; double eff; };
+  struct Cand { int v; double eff; };
   // with two m/n-contiguous operands (RS) the hand-scheduled tiles gain less over the 256x256 ring than with a
   // k-contiguous operand, and the 192-wide ring tiles do best on four 32-deep stages
   const bool rs = p.flow == RS;
-  const Cand cands[] = {{1, 256, 256, 1.0},                    {10, 256, 384, rs ? 1.02 : 1.06}, {11, 384, 192, rs ? 0.96 : 1.04},
-                        {rs ? 5 : 8, 256, 192, rs ? 0.95 : 0.93}, {rs ? 6 : 9, 192, 256, rs ? 0.95 : 0.93}, {3, 128, 128, 0.55}};
+  const Cand cands[] = {{1, 1.0}, {10, rs ? 1.02 : 1.06}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, 0.55}};
   const long chunks = p.flow == OS ? 1 : p.S;
-  Pick best = {0, 0};
+  const double total_k = (double)p.K * p.S;
+  Pick best = {0, 1, 0};
   for (const Cand &c : cands) {
-    const long tiles = (long)((p.M + c.bm - 1) / c.bm) * ((p.N + c.bn - 1) / c.bn) * chunks;
-    const long rounds = (tiles + dev.cus - 1) / dev.cus;
-    const double cost = (double)rounds * c.bm * c.bn / c.eff;
-    if (best.v == 0 || cost < best.cost) best = {c.v, cost};
+    const int bm = TILE_OF[c.v].bm, bn = TILE_OF[c.v].bn;
+    const long tiles = (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn) * chunks;
+    for (int splits : SPLIT_CHOICES) {
+      if (g_splits != 0 && splits != g_splits) continue;
+      if (splits > 1 && (split_refused(p, dev, c.v, splits) || (g_splits == 0 && total_k / splits < SPLIT_MIN_K))) continue;
+      const long rounds = (tiles * splits + dev.cus - 1) / dev.cus;
+      const double exchange = splits == 1 ? 0.0 : (SPLIT_FIX + (double)splits * p.M * p.N * SPLIT_PER_ELEMENT) / total_k;
+      const double cost = (double)rounds * bm * bn / c.eff / splits + exchange;
+      if (best.v == 0 || cost < best.cost) best = {c.v, splits, cost};
+    }
   }
   return best;
 }
 
-int launch_variant(int v, const Problem &p, const DevInfo &dev, hipStream_t stream) {
+int launch_variant(int v, int splits, const Problem &p, const DevInfo &dev, hipStream_t stream) {
+  if (g_launches == 0) { g_last_variant = v; g_last_splits = splits; }
   switch (v) {
-    case 1: return launch_bf16_tile<256, 256, 2, 2, 64, 2>(p, dev, stream);
-    case 2: return launch_bf16_tile<256, 256, 2, 4, 32, 4>(p, dev, stream);
-    case 3: return launch_bf16_tile<128, 128, 2, 2, 64, 2>(p, dev, stream);
-    case 4: return launch_bf16_tile<256, 256, 2, 2, 32, 4>(p, dev, stream);
-    case 5: return launch_bf16_tile<256, 192, 2, 2, 32, 4>(p, dev, stream);
-    case 6: return launch_bf16_tile<192, 256, 2, 2, 32, 4>(p, dev, stream);
-    case 7: return launch_bf16_tile<256, 256, 2, 4, 64, 2>(p, dev, stream);
-    case 8: return launch_bf16_tile<256, 192, 2, 2, 64, 2>(p, dev, stream);
-    case 9: return launch_bf16_tile<192, 256, 2, 2, 64, 2>(p, dev, stream);
-    case 10: return launch_bf16_tile<256, 384, 2, 2, 64, 2, true>(p, dev, stream);
-    case 11: return launch_bf16_tile<384, 192, 2, 2, 64, 2, true>(p, dev, stream);
+    case 1: return launch_bf16_tile<256, 256, 2, 2, 64, 2>(p, dev, stream, 1, splits);
+    case 2: return launch_bf16_tile<256, 256, 2, 4, 32, 4>(p, dev, stream, 2, splits);
+    case 3: return launch_bf16_tile<128, 128, 2, 2, 64, 2>(p, dev, stream, 3, splits);
+    case 4: return launch_bf16_tile<256, 256, 2, 2, 32, 4>(p, dev, stream, 4, splits);
+    case 5: return launch_bf16_tile<256, 192, 2, 2, 32, 4>(p, dev, stream, 5, splits);
+    case 6: return launch_bf16_tile<192, 256, 2, 2, 32, 4>(p, dev, stream, 6, splits);
+    case 7: return launch_bf16_tile<256, 256, 2, 4, 64, 2>(p, dev, stream, 7, splits);
+    case 8: return launch_bf16_tile<256, 192, 2, 2, 64, 2>(p, dev, stream, 8, splits);
+    case 9: return launch_bf16_tile<192, 256, 2, 2, 64, 2>(p, dev, stream, 9, splits);
+    case 10: return launch_bf16_tile<256, 384, 2, 2, 64, 2, true>(p, dev, stream, 10, splits);
+    case 11: return launch_bf16_tile<384, 192, 2, 2, 64, 2, true>(p, dev, stream, 11, splits);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }
@@ -261,9 +340,9 @@ int launch_variant(int v, const Problem &p, const DevInfo &dev, hipStream_t stre
 // their chunks are promised in slice order.
 int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
-  if (g_variant != 0) return launch_variant(g_variant, p, dev, stream);
+  if (g_variant != 0) return launch_variant(g_variant, g_splits > 1 ? g_splits : 1, p, dev, stream);
   const Pick single = pick_variant(p, dev);
-  if (p.flow == OS) {
+  if (p.flow == OS && single.splits == 1 && g_splits == 0) {
     constexpr int BM = 256, BN = 384;
     constexpr double EFF = 1.06;
     const long tiles_m = (p.M + BM - 1) / BM;
@@ -275,6 +354,7 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
     if (nb1 > 0 && n1 < p.N) {
       Problem rest = p;
       rest.N = p.N - (int)n1;
+      rest.ws = nullptr;   // the second launch is not split: the first may still be using the workspace's counters
       const Pick tail = pick_variant(rest, dev);
       const double second_launch = 3.4e7 / (double)total_k;      // ~12 us at the rate one CU computes tile area x K
       const double cost = (double)(tiles_m * nb1 / dev.cus) * BM * BN / EFF + tail.cost + second_launch;
@@ -282,7 +362,7 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
         const int es_in = 2, es_out = p.out_dtype == MS_DTYPE_BF16 ? 2 : 4;
         Problem head = p;
         head.N = (int)n1;
-        int rc = launch_variant(10, head, dev, stream);
+        int rc = launch_variant(10, 1, head, dev, stream);
         if (rc != MS_OK) return rc;
         const void *b2[MS_MAX_SLICES];
         void *c2[1] = {static_cast<char *>(p.c[0]) + n1 * es_out};
@@ -290,11 +370,11 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
         rest.b = b2;
         rest.c = c2;
         if (p.res) rest.res = static_cast<const char *>(p.res) + n1 * es_out;
-        return launch_variant(tail.v, rest, dev, stream);
+        return launch_variant(tail.v, 1, rest, dev, stream);
       }
     }
   }
-  return launch_variant(single.v, p, dev, stream);
+  return launch_variant(single.v, single.splits, p, dev, stream);
 }
 
 int launch_f32(const Problem &p, hipStream_t stream) {
@@ -331,6 +411,8 @@ int run(const Problem &p, void *stream) {
   if (rc) return rc;
   hipStream_t st = (hipStream_t)stream;
   g_launches = 0;
+  g_last_variant = 0;
+  g_last_splits = 1;
   return p.in_dtype == MS_DTYPE_BF16 ? launch_bf16(p, *dev, st) : launch_f32(p, st);
 }
 
@@ -390,6 +472,8 @@ MS_API const char *ms_last_error(void) { return g_err; }
 MS_API long ms_query(int what) {
   if (what == MS_QUERY_MAX_SLICES) return MS_MAX_SLICES;
   if (what == MS_QUERY_LAST_LAUNCHES) return g_launches;
+  if (what == MS_QUERY_LAST_VARIANT) return g_last_variant;
+  if (what == MS_QUERY_LAST_SPLITS) return g_last_splits;
   DevInfo *d = nullptr;
   if (dev_info(&d) != MS_OK) return -1;
   switch (what) {
@@ -402,8 +486,33 @@ MS_API long ms_query(int what) {
 }
 
 MS_API int ms_set_variant(int variant) {
-  if (variant < 0 || variant > 11) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
-  g_variant = variant;
+  const int v = variant % 100, splits = variant / 100;
+  if (variant < 0 || v > VARIANTS || splits == 1 || splits > SPLIT_MAX) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  g_variant = v;
+  g_splits = splits;
+  return MS_OK;
+}
+
+namespace {
+__global__ void ws_clear_kernel(int *counters, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) counters[i] = 0;
+}
+}  // namespace
+
+MS_API size_t ms_workspace_bytes(void) {
+  DevInfo *d = nullptr;
+  if (dev_info(&d) != MS_OK) return 0;
+  // one partial tile of the largest shape (256 x 384 fp32) per compute unit
+  return WS_HEADER_BYTES + (size_t)d->cus * 256 * 384 * sizeof(float);
+}
+
+MS_API int ms_workspace_init(void *workspace, size_t bytes, void *stream) {
+  if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) || bytes < WS_HEADER_BYTES)
+    return fail(MS_ERR_ARG, "ms_workspace_init: a workspace must be 256-byte aligned and hold at least %zu bytes", WS_HEADER_BYTES);
+  // a fill kernel, not hipMemsetAsync, so that the call may be captured into a HIP graph
+  hipLaunchKernelGGL(ws_clear_kernel, dim3(WS_COUNTERS / 256), dim3(256), 0, (hipStream_t)stream, static_cast<int *>(workspace), WS_COUNTERS);
+  MS_HIP(hipGetLastError());
   return MS_OK;
 }
 
@@ -419,6 +528,17 @@ MS_API int ms_gemm_os_fused(const void *const *A_slices, const void *const *B_sl
   void *c1[1] = {C};
   Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
   p.act = activation; p.res = residual; p.ldr = ldr; p.row_sum = row_sum; p.row_sumsq = row_sumsq;
+  return run(p, stream);
+}
+
+MS_API int ms_gemm_os_ws(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
+                         int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype, int activation,
+                         const void *residual, int ldr, float *row_sum, float *row_sumsq,
+                         void *workspace, size_t workspace_bytes, void *stream) {
+  void *c1[1] = {C};
+  Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
+  p.act = activation; p.res = residual; p.ldr = ldr; p.row_sum = row_sum; p.row_sumsq = row_sumsq;
+  p.ws = workspace; p.ws_bytes = workspace ? workspace_bytes : 0;
   return run(p, stream);
 }
 
@@ -451,6 +571,15 @@ MS_API int ms_time_os(const void *const *A_slices, const void *const *B_slices, 
                       int warmup, int reps, float *ms_out) {
   void *c1[1] = {C};
   return timed(make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype), stream, warmup, reps, ms_out);
+}
+
+MS_API int ms_time_os_ws(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
+                         int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype,
+                         void *workspace, size_t workspace_bytes, void *stream, int warmup, int reps, float *ms_out) {
+  void *c1[1] = {C};
+  Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
+  p.ws = workspace; p.ws_bytes = workspace ? workspace_bytes : 0;
+  return timed(p, stream, warmup, reps, ms_out);
 }
 
 MS_API int ms_time_ls_ex(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,

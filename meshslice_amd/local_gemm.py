@@ -45,6 +45,38 @@ def _same(ts: Sequence[torch.Tensor], name: str):
     return s0
 
 
+_workspaces = {}
+
+
+def workspace(device) -> torch.Tensor:
+    """The split-contraction workspace of ``device`` (a uint8 tensor of ``ms_workspace_bytes()`` bytes, allocated and
+    prepared with ``ms_workspace_init`` on first use, then kept): ``gemm_os`` hands it to ``ms_gemm_os_ws`` so that
+    products with few output tiles can spread their contraction over the idle compute units.  Calls that use it
+    must not overlap on the device (they share its counters): issue them on one stream, or order them with events."""
+    device = torch.device(device)
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    ws = _workspaces.get(idx)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise _lib.MeshSliceError("the workspace of this device does not exist yet and cannot be allocated while a "
+                                      "graph is being captured: call gemm_os (or local_gemm.workspace) once before the capture")
+        lib = _lib.load()
+        with torch.cuda.device(idx):
+            nbytes = int(lib.ms_workspace_bytes())
+            if nbytes <= 0:
+                raise _lib.MeshSliceError("could not size the workspace: " + _lib.last_error())
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=torch.device("cuda", idx))
+            _lib.check(lib.ms_workspace_init(ctypes.c_void_p(ws.data_ptr()), nbytes, _stream()))
+            torch.cuda.current_stream().synchronize()     # later calls may come on any stream
+        _workspaces[idx] = ws
+    return ws
+
+
+def _ws_args(device):
+    ws = workspace(device)
+    return ctypes.c_void_p(ws.data_ptr()), ws.numel()
+
+
 class _Call:
     """One validated local contraction: the C entry points' argument list up to (not including) ``stream``,
     the device it runs on, the output it writes and the Python objects that keep the pointer tables alive."""
@@ -120,12 +152,6 @@ def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
     call = _prepare_os(A_slices, B_slices, out, out_dtype)
     out = call.out
     m, n = out.shape
-    fused = activation is not None or residual is not None or row_moments is not None
-    if not fused:
-        with torch.cuda.device(call.device):
-            rc = _lib.load().ms_gemm_os(*call.args, _stream())
-        _lib.check(rc)
-        return out
     if activation not in (None, "gelu"):
         raise ValueError(f"unknown activation {activation!r} (None or 'gelu')")
     res_ptr, ldr = None, 0
@@ -141,10 +167,11 @@ def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
                     and t.device == out.device):
                 raise ValueError("row moments must be contiguous fp32 GPU vectors of length m on the output's device")
             moments[idx] = ctypes.c_void_p(t.data_ptr())
+    ws_ptr, ws_bytes = _ws_args(call.device)
     with torch.cuda.device(call.device):
-        rc = _lib.load().ms_gemm_os_fused(*call.args,
-                                          _lib.MS_ACT_GELU if activation == "gelu" else _lib.MS_ACT_NONE,
-                                          res_ptr, ldr, moments[0], moments[1], _stream())
+        rc = _lib.load().ms_gemm_os_ws(*call.args,
+                                       _lib.MS_ACT_GELU if activation == "gelu" else _lib.MS_ACT_NONE,
+                                       res_ptr, ldr, moments[0], moments[1], ws_ptr, ws_bytes, _stream())
     _lib.check(rc)
     return out
 
@@ -197,7 +224,13 @@ def time_call(flow: str, operands, out, warmup: int = 5, reps: int = 20) -> List
     first, second = operands
     lib = _lib.load()
     if flow == "os":
-        call, fn = _prepare_os(first, second, out, None), lib.ms_time_os
+        call = _prepare_os(first, second, out, None)
+        ms = (ctypes.c_float * int(reps))()
+        ws_ptr, ws_bytes = _ws_args(call.device)
+        with torch.cuda.device(call.device):
+            rc = lib.ms_time_os_ws(*call.args, ws_ptr, ws_bytes, _stream(), int(warmup), int(reps), ms)
+        _lib.check(rc)
+        return list(ms)
     elif flow == "ls":
         call, fn = _prepare_ls(first, second, out, None), lib.ms_time_ls_ex
     else:

@@ -1,0 +1,160 @@
+"""Output-stationary products whose contraction is split over compute units (``ms_gemm_os_ws``): parity with the
+float64 oracle and with the unsplit kernels, run-to-run bit-identity, the fused epilogue, HIP-graph capture, the
+workspace rules of the C ABI.  Tolerance: rel-Frobenius <= 1e-2 against the oracle (bf16 in, fp32 accumulate)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import meshslice_oracle as orc
+import meshslice_amd as ms
+from meshslice_amd import _lib, local_gemm
+
+pytestmark = pytest.mark.gpu
+TOL_BF16 = 1e-2
+SPLIT_VARIANTS = (2, 3, 5, 6, 7, 8, 9, 10, 11)      # 1 and 4 (256x256 on four waves) have no split path
+
+
+@pytest.fixture(autouse=True)
+def _default_variant():
+    _lib.load().ms_set_variant(0)
+    yield
+    _lib.load().ms_set_variant(0)
+    torch.cuda.synchronize()
+
+
+def _rand(shape, scale, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (torch.randn(shape, generator=g, device="cuda") * scale).to(torch.bfloat16)
+
+
+def _f64(t):
+    return t.float().cpu().numpy().astype(np.float64)
+
+
+def _counters():
+    ws = local_gemm.workspace("cuda")
+    return ws[:4096].view(torch.int32)
+
+
+@pytest.mark.parametrize("variant", SPLIT_VARIANTS)
+@pytest.mark.parametrize("splits", [2, 3, 8])
+def test_forced_split_matches_oracle_and_is_bit_reproducible(variant, splits):
+    """Ragged shapes (edge tiles, a K tail, K steps that do not divide by the split count, slices that a split's
+    K range crosses) on every tile variant that can split."""
+    L = _lib.load()
+    m, n, ks, S = 200, 424, 712, 3             # 3 slices of 712 = 11.1 K steps of 64 each
+    A = [_rand((m, ks), 1.0, 10 + s) for s in range(S)]
+    B = [_rand((ks, n), 0.05, 20 + s) for s in range(S)]
+    want = sum(_f64(a) @ _f64(b) for a, b in zip(A, B))
+    L.ms_set_variant(variant)
+    plain = ms.gemm_os(A, B, out_dtype=torch.float32)
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+    L.ms_set_variant(variant + 100 * splits)
+    got = ms.gemm_os(A, B, out_dtype=torch.float32)
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == splits and L.ms_query(_lib.MS_QUERY_LAST_VARIANT) == variant
+    assert orc.rel_frobenius(_f64(got), want) <= 1e-5 * 50      # fp32 out of bf16 operands: accumulation error only
+    assert orc.rel_frobenius(_f64(got), _f64(plain)) <= 1e-6
+    for _ in range(3):                                          # the sum order is fixed: same bits every time
+        assert torch.equal(ms.gemm_os(A, B, out_dtype=torch.float32), got)
+    torch.cuda.synchronize()
+    assert int(_counters().abs().sum()) == 0                    # the arrival counters are clear again
+    out_bf16 = ms.gemm_os(A, B)
+    assert torch.equal(out_bf16, got.to(torch.bfloat16))        # bf16 output = one rounding of the same sums
+
+
+def test_small_output_long_contraction_is_split_by_default():
+    """2048 x 1536 x 12288 (out_proj backward-data on an 8x8 mesh): 64 tiles for 256 compute units."""
+    L = _lib.load()
+    A = [_rand((2048, 3072), 1.0, 30 + s) for s in range(4)]
+    B = [_rand((3072, 1536), 0.02, 40 + s) for s in range(4)]
+    C = ms.gemm_os(A, B)
+    splits = L.ms_query(_lib.MS_QUERY_LAST_SPLITS)
+    assert splits > 1
+    rows = np.random.default_rng(0).choice(2048, 64, replace=False)
+    want = sum(_f64(a[rows]) @ _f64(b) for a, b in zip(A, B))
+    assert orc.rel_frobenius(_f64(C[rows]), want) <= TOL_BF16
+    assert torch.equal(ms.gemm_os(A, B), C)
+    # the same product without a workspace is not split and agrees to output rounding
+    pa, _ka = _lib.ptr_array([t.data_ptr() for t in A]); pb, _kb = _lib.ptr_array([t.data_ptr() for t in B])
+    C1 = torch.empty_like(C)
+    rc = L.ms_gemm_os(pa, pb, 4, 2048, 1536, 3072, 3072, 1536, ctypes.c_void_p(C1.data_ptr()), 1536,
+                      _lib.MS_DTYPE_BF16, _lib.MS_DTYPE_BF16, None)
+    assert rc == 0 and L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+    assert orc.rel_frobenius(_f64(C1), _f64(C)) <= 4e-3
+    # a product with a tile per compute unit (or more) stays unsplit
+    ms.gemm_os([_rand((4096, 1024), 1.0, 1)], [_rand((1024, 12288), 0.02, 2)])
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+
+
+def test_a_fused_epilogue_keeps_the_product_unsplit():
+    """The fused-epilogue kernels carry no exchange of partial tiles: a product that would split runs unsplit when an
+    epilogue is asked for, and a forced split is refused."""
+    L = _lib.load()
+    A = [_rand((2048, 3072), 1.0, 30 + s) for s in range(4)]
+    B = [_rand((3072, 1536), 0.02, 40 + s) for s in range(4)]
+    plain = ms.gemm_os(A, B, out_dtype=torch.float32)
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) > 1
+    fused = ms.gemm_os(A, B, out_dtype=torch.float32, activation="gelu")
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+    assert orc.rel_frobenius(_f64(fused), orc.gelu_tanh(_f64(plain))) <= 1e-5
+    L.ms_set_variant(408)
+    with pytest.raises(ValueError, match="fused epilogue"):
+        ms.gemm_os(A, B, activation="gelu")
+
+
+def test_split_product_replays_from_a_hip_graph():
+    A = [_rand((1024, 2048), 1.0, 60 + s) for s in range(2)]
+    B = [_rand((2048, 1536), 0.02, 70 + s) for s in range(2)]
+    out = torch.empty((1024, 1536), dtype=torch.bfloat16, device="cuda")
+    eager = ms.gemm_os(A, B)
+    assert _lib.load().ms_query(_lib.MS_QUERY_LAST_SPLITS) > 1
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ms.gemm_os(A, B, out=out)
+    for _ in range(3):
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        assert torch.equal(ms.gemm_os(A, B), eager)     # eager work between the replays
+
+
+def test_workspace_rules_of_the_c_abi():
+    L = _lib.load()
+    A = _rand((256, 2048), 1.0, 80); B = _rand((2048, 256), 0.05, 81)
+    C = torch.empty((256, 256), dtype=torch.bfloat16, device="cuda")
+    pa, _ka = _lib.ptr_array([A.data_ptr()]); pb, _kb = _lib.ptr_array([B.data_ptr()])
+    head = (pa, pb, 1, 256, 256, 2048, 2048, 256, ctypes.c_void_p(C.data_ptr()), 256, _lib.MS_DTYPE_BF16, _lib.MS_DTYPE_BF16)
+    epi = (_lib.MS_ACT_NONE, None, 0, None, None)
+    ws = local_gemm.workspace("cuda")
+    assert ws.numel() == L.ms_workspace_bytes() >= 4096 + 256 * 256 * 384 * 4 // 2
+    # no workspace: the product runs unsplit; a forced split is refused
+    assert L.ms_gemm_os_ws(*head, *epi, None, 0, None) == 0 and L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+    L.ms_set_variant(408)
+    assert L.ms_gemm_os_ws(*head, *epi, None, 0, None) == _lib.MS_ERR_ARG
+    assert "workspace" in _lib.last_error()
+    # misaligned or undersized workspaces are argument errors
+    assert L.ms_gemm_os_ws(*head, *epi, ctypes.c_void_p(ws.data_ptr() + 16), 1 << 20, None) == _lib.MS_ERR_ARG
+    assert L.ms_gemm_os_ws(*head, *epi, ctypes.c_void_p(ws.data_ptr()), 1024, None) == _lib.MS_ERR_ARG
+    # a workspace too small for the partial tiles of a forced split is refused with the reason
+    assert L.ms_gemm_os_ws(*head, *epi, ctypes.c_void_p(ws.data_ptr()), 4096 + 1000, None) == _lib.MS_ERR_ARG
+    assert "do not fit" in _lib.last_error()
+    # ... and merely narrows the library's own choice
+    L.ms_set_variant(0)
+    assert L.ms_gemm_os_ws(*head, *epi, ctypes.c_void_p(ws.data_ptr()), 4096 + 1000, None) == 0
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+    # variants without a split path refuse (256x256 on four waves); bad split counts are unknown variants
+    L.ms_set_variant(401)
+    assert L.ms_gemm_os_ws(*head, *epi, ctypes.c_void_p(ws.data_ptr()), ws.numel(), None) == _lib.MS_ERR_ARG
+    assert "no split path" in _lib.last_error()
+    assert L.ms_set_variant(108) == _lib.MS_ERR_ARG and L.ms_set_variant(908) == _lib.MS_ERR_ARG and L.ms_set_variant(12) == _lib.MS_ERR_ARG
+    L.ms_set_variant(0)
+    assert L.ms_workspace_init(None, 4096, None) == _lib.MS_ERR_ARG
+    assert L.ms_workspace_init(ctypes.c_void_p(ws.data_ptr()), 100, None) == _lib.MS_ERR_ARG
+    torch.cuda.synchronize()
+    got = ms.gemm_os([A], [B])
+    assert orc.rel_frobenius(_f64(got), _f64(A) @ _f64(B)) <= TOL_BF16
