@@ -110,6 +110,17 @@ int ms_gemm_os_ws(const void *const *A_slices, const void *const *B_slices, int 
                   float *row_sum, float *row_sumsq,
                   void *workspace, size_t workspace_bytes, void *stream);
 
+/* ms_gemm_os_ws (plain product) for callers that cannot allocate device memory or be handed a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  The
+ * split-contraction workspace is a fixed array inside the library's code object (4096 + 48 MiB per device, held until the
+ * process ends); the call allocates and frees nothing.  A product whose exchange of partial tiles would not fit that
+ * array is refused with MS_ERR_UNSUPPORTED (the message names the sizes) — use ms_gemm_os_ws there.  All calls on one
+ * device share the array: calls that overlap on a device (different streams without an ordering between them, several
+ * host threads) race on it and give wrong results; issue them on one stream or order them with events. */
+int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_slices, int S,
+                       int m, int n, int k_slice, int lda, int ldb,
+                       void *C, int ldc, int in_dtype, int out_dtype, void *stream);
+
 /* Bytes of workspace that let every product split its contraction on the current device (0 on a HIP error). */
 size_t ms_workspace_bytes(void);
 

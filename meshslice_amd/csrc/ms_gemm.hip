@@ -493,7 +493,32 @@ MS_API int ms_set_variant(int variant) {
   return MS_OK;
 }
 
+// Scratch of the entry point that allocates nothing (ms_gemm_os_noalloc): a split-contraction workspace that lives in
+// the code object.  Every device the library runs on holds its own copy, at its own address, until the process ends; the
+// name below is only a handle for hipGetSymbolAddress, host code never passes it to a kernel.
+constexpr size_t NOALLOC_SCRATCH_BYTES = WS_HEADER_BYTES + (size_t)256 * 256 * 192 * sizeof(float);   // 256 partial tiles of 256 x 192
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
 namespace {
+struct ScratchAddr {
+  std::once_flag once;
+  hipError_t err = hipSuccess;
+  void *ptr = nullptr;
+};
+ScratchAddr g_scratch[64];
+
+// Device address of `scratch` on the calling thread's current device, looked up once per device with that device current.
+int scratch_address(void **out) {
+  int d = 0;
+  MS_HIP(hipGetDevice(&d));
+  if (d < 0 || d >= 64) return fail(MS_ERR_HIP, "device ordinal %d out of range", d);
+  ScratchAddr &sa = g_scratch[d];
+  std::call_once(sa.once, [&sa]() { sa.err = hipGetSymbolAddress(&sa.ptr, HIP_SYMBOL(scratch)); });
+  if (sa.err != hipSuccess || !sa.ptr) return fail(MS_ERR_HIP, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(sa.err));
+  *out = sa.ptr;
+  return MS_OK;
+}
+
 __global__ void ws_clear_kernel(int *counters, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) counters[i] = 0;
@@ -539,6 +564,41 @@ MS_API int ms_gemm_os_ws(const void *const *A_slices, const void *const *B_slice
   Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
   p.act = activation; p.res = residual; p.ldr = ldr; p.row_sum = row_sum; p.row_sumsq = row_sumsq;
   p.ws = workspace; p.ws_bytes = workspace ? workspace_bytes : 0;
+  return run(p, stream);
+}
+
+MS_API int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
+                              int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype, void *stream) {
+  void *c1[1] = {C};
+  Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
+  int rc = validate(p);
+  if (rc) return rc;
+  if (in_dtype == MS_DTYPE_BF16) {
+    DevInfo *dev = nullptr;
+    rc = dev_info(&dev);
+    if (rc) return rc;
+    // what the library would do with room to spare decides whether the built-in scratch is enough
+    p.ws = reinterpret_cast<void *>(uintptr_t(256));    // stands for "a workspace": only its size is looked at here
+    p.ws_bytes = ~size_t(0);
+    const Pick want = g_variant != 0 ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, *dev);
+    if (want.splits > 1) {
+      const TileShape t = TILE_OF[want.v];
+      const size_t tiles = (size_t)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
+      const size_t need = WS_HEADER_BYTES + tiles * want.splits * t.bm * t.bn * sizeof(float);
+      if (need > NOALLOC_SCRATCH_BYTES)
+        return fail(MS_ERR_UNSUPPORTED, "ms_gemm_os_noalloc: this product (m=%d n=%d k=%d x %d slices) would exchange %zu bytes of partial "
+                    "tiles, the built-in scratch holds %zu; use ms_gemm_os_ws with a workspace of ms_workspace_bytes()",
+                    m, n, k_slice, S, need, NOALLOC_SCRATCH_BYTES);
+    }
+    void *ptr = nullptr;
+    rc = scratch_address(&ptr);
+    if (rc) return rc;
+    p.ws = ptr;
+    p.ws_bytes = NOALLOC_SCRATCH_BYTES;
+    // the array keeps what the last call left: the counters must start at zero (a fill kernel, so that the call can be captured)
+    hipLaunchKernelGGL(ws_clear_kernel, dim3(WS_COUNTERS / 256), dim3(256), 0, (hipStream_t)stream, static_cast<int *>(ptr), WS_COUNTERS);
+    MS_HIP(hipGetLastError());
+  }
   return run(p, stream);
 }
 
