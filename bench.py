@@ -102,6 +102,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 1 GiB device copy (scales rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--only-main", action="store_true", help="skip the S=1 / LS / RS side measurements")
+    ap.add_argument("--kernel-only", choices=("os", "ls", "rs"), default=None,
+                    help="profiling runs: launch only the kernel of configuration 2 (os), 3 (ls) or 4 (rs) and print its time")
+    ap.add_argument("--variant", type=int, default=0, help="profiling runs: force a bf16 kernel variant (ms_set_variant), 0 = library's choice")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE mesh device's local GEMM on ONE GPU; --gpus > 1 is not part of this build "
@@ -130,6 +133,38 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.variant:
+        _lib.check(lib.ms_set_variant(args.variant))
+
+    if args.kernel_only:
+        # one configuration's kernel alone, for the profiler: settle + warm-up + steps back-to-back launches
+        if args.kernel_only == "os":
+            run, fl = (lambda: ms.gemm_os(A, B, out=C)), flops
+        elif args.kernel_only == "ls":
+            Ws = [W[torch.from_numpy(sel_index(12288, 8, 8, k)).cuda(), :].contiguous() for k in range(8)]
+            Y = [torch.empty((4096, 1536), dtype=torch.float32, device="cuda") for _ in range(8)]
+            run, fl = (lambda: ms.gemm_ls(X, Ws, out=Y)), flops
+        else:
+            g = torch.Generator(device="cuda").manual_seed(4)
+            X4 = torch.randn((4096, 3072), generator=g, device="cuda").to(torch.bfloat16)
+            dY = (torch.randn((4096, 12288), generator=g, device="cuda") * 1e-3).to(torch.bfloat16)
+            Xs = [X4[:, torch.from_numpy(sel_index(3072, 4, 8, k)).cuda()].contiguous() for k in range(4)]
+            Y = [torch.empty((768, 12288), dtype=torch.float32, device="cuda") for _ in range(4)]
+            run, fl = (lambda: ms.gemm_rs(Xs, dY, out=Y)), 2.0 * 3072 * 12288 * 4096
+        for _ in range(SETTLE_LAUNCHES + args.warmup):
+            run()
+        e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            run()
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) / args.steps
+        print(json.dumps({"kernel_only": args.kernel_only, "kernel_variant": int(lib.ms_query(_lib.MS_QUERY_LAST_VARIANT)),
+                          "splits": int(lib.ms_query(_lib.MS_QUERY_LAST_SPLITS)), "steps": args.steps, "kernel_ms_mean": round(t, 4),
+                          "tflops": round(fl / t / 1e9, 1), "frac_of_bf16_peak": round(fl / t / 1e9 / PEAK_BF16_TFLOPS, 4)}), flush=True)
+        return
 
     # ---- settle phase (always, whatever --warmup says): the first launches after an idle period run up to 30 % slow
     for _ in range(SETTLE_LAUNCHES):

@@ -11,6 +11,7 @@
 
 #include "ms_gemm_bf16.hip.inc"
 #include "ms_gemm_bf16_big.hip.inc"
+#include "ms_gemm_bf16_x16.hip.inc"
 #include "ms_gemm_f32.hip.inc"
 
 // Every kernel variant is instantiated explicitly: with implicit instantiation alone the host
@@ -46,6 +47,14 @@ MS_INSTANTIATE_RING(192, 256, 64, 2, 2, 2)
 MS_INSTANTIATE_BIG(4, 6)
 MS_INSTANTIATE_BIG(6, 3)
 #undef MS_INSTANTIATE_BIG
+template __global__ void msk::gemm_bf16_x16_kernel<true, false, true, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_x16_kernel<true, false, false, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_x16_kernel<true, false, true, true>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_x16_kernel<true, false, false, true>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_x16_kernel<true, true, false, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_x16_kernel<true, true, true, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_x16_kernel<false, false, false, false>(const msk::GemmArgs);
+template __global__ void msk::gemm_bf16_x16_kernel<false, false, true, false>(const msk::GemmArgs);
 
 namespace {
 thread_local char g_err[512] = "";
@@ -169,14 +178,18 @@ int validate(const Problem &p) {
   return MS_OK;
 }
 
-// BIG = false: gemm_bf16_ring_kernel<BM, BN, ...>; BIG = true: gemm_bf16_big_kernel (256x384x64, 2x2 waves, two stages)
-template <bool BIG, int BM, int BN, int BK_, int NS, int WGM, int WGN, bool AK, bool BKM, bool OBF, bool EPI>
+// KIND 0: gemm_bf16_ring_kernel<BM, BN, ...>; 1: gemm_bf16_big_kernel (32x32x16 MFMA, 2x2 waves, two 64-deep stages);
+// 2: gemm_bf16_x16_kernel (256x384x64 on the 16x16x32 MFMA)
+template <int KIND, int BM, int BN, int BK_, int NS, int WGM, int WGN, bool AK, bool BKM, bool OBF, bool EPI>
 void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
-  if constexpr (!BIG) {
+  if constexpr (KIND == 0) {
     msk::gemm_bf16_ring_kernel<BM, BN, BK_, NS, WGM, WGN, AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
-  } else {
+  } else if constexpr (KIND == 1) {
     static_assert(BM % 64 == 0 && BN % 64 == 0 && BK_ == 64 && NS == 2 && WGM == 2 && WGN == 2, "the big-tile kernels are 2 x 2 waves on two 64-deep stages");
     msk::gemm_bf16_big_kernel<BM / 64, BN / 64, AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
+  } else {
+    static_assert(BM == 256 && BN == 384 && BK_ == 64 && NS == 2 && WGM == 2 && WGN == 2, "the 16x16x32 kernel has one shape");
+    msk::gemm_bf16_x16_kernel<AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
   }
 }
 
@@ -184,7 +197,7 @@ extern const char *const SPLIT_REFUSALS[];
 int split_refused(const Problem &p, const DevInfo &dev, int variant, int splits);
 
 // tile BM x BN, WGM x WGN waves, NS ring stages of BK_ k-elements; contraction split `splits` ways
-template <int BM, int BN, int WGM, int WGN, int BK_, int NS, bool BIG = false>
+template <int BM, int BN, int WGM, int WGN, int BK_, int NS, int KIND = 0>
 int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream, int variant, int splits) {
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
@@ -219,18 +232,18 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream, i
   const bool epi = p.act != 0 || p.res || p.row_sum || p.row_sumsq;
   if (p.flow == OS) {
     if (epi) {
-      if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, true, true>(gd, bd, stream, g);
-      else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, false, true>(gd, bd, stream, g);
+      if (obf) launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, true, false, true, true>(gd, bd, stream, g);
+      else launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, true, false, false, true>(gd, bd, stream, g);
     } else {
-      if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, true, false>(gd, bd, stream, g);
-      else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, false, false, false>(gd, bd, stream, g);
+      if (obf) launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, true, false, true, false>(gd, bd, stream, g);
+      else launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, true, false, false, false>(gd, bd, stream, g);
     }
   } else if (p.flow == LS) {
-    if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, true, true, false>(gd, bd, stream, g);
-    else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, true, true, false, false>(gd, bd, stream, g);
+    if (obf) launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, true, true, true, false>(gd, bd, stream, g);
+    else launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, true, true, false, false>(gd, bd, stream, g);
   } else {
-    if (obf) launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, false, false, true, false>(gd, bd, stream, g);
-    else launch_one<BIG, BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
+    if (obf) launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, false, false, true, false>(gd, bd, stream, g);
+    else launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
   }
   g_launches++;
   MS_HIP(hipGetLastError());
@@ -242,6 +255,7 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream, i
 //   4: 256x256, 4 waves, 4 x 32     5: 256x192, 4 waves, 4 x 32     6: 192x256, 4 waves, 4 x 32
 //   7: 256x256, 8 waves, 2 x 64     8: 256x192, 4 waves, 2 x 64     9: 192x256, 4 waves, 2 x 64
 //  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel<4, 6>)     11: 384x192, 4 waves, 2 x 64 (gemm_bf16_big_kernel<6, 3>)
+//  12: 256x384, 4 waves, 2 x 64 on the 16x16x32 MFMA (gemm_bf16_x16_kernel)
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
 // ceil(work items / CUs) rounds of one item per CU, so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile reaches 1.06
@@ -257,10 +271,11 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream, i
 // 2048 x 1536 x 12288 (64 tiles of 256x192): 170 us unsplit, 100 / 85 / 88 us with 2 / 3 / 4 splits.
 struct Pick { int v, splits; double cost; };
 
-constexpr int VARIANTS = 11;
+constexpr int VARIANTS = 12;
 struct TileShape { int bm, bn; };
 constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256}, {128, 128}, {256, 256}, {256, 192},
-                                             {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192}};
+                                             {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192},
+                                             {256, 384}};
 constexpr int SPLIT_CHOICES[] = {1, 2, 3, 4, 6, 8};
 constexpr int SPLIT_MAX = 8;
 constexpr long SPLIT_MIN_K = 512;            // contraction elements per split item, at least
@@ -277,7 +292,7 @@ const char *const SPLIT_REFUSALS[] = {"", "only output-stationary products split
 int split_refused(const Problem &p, const DevInfo &dev, int v, int splits) {
   const int bm = TILE_OF[v].bm, bn = TILE_OF[v].bn;
   if (splits < 2 || splits > SPLIT_MAX) return 7;
-  if (v == 1 || v == 4) return 8;     // 256x256 on four waves: see ring_can_split
+  if (v == 1 || v == 4 || v == 12) return 8;     // 256x256 on four waves: see ring_can_split; the 16x16x32 kernel has none
   if (p.act || p.res || p.row_sum || p.row_sumsq) return 9;   // see ring_can_split, big_can_split
   if (p.flow != OS) return 1;
   if (!p.ws) return 2;
@@ -326,8 +341,9 @@ int launch_variant(int v, int splits, const Problem &p, const DevInfo &dev, hipS
     case 7: return launch_bf16_tile<256, 256, 2, 4, 64, 2>(p, dev, stream, 7, splits);
     case 8: return launch_bf16_tile<256, 192, 2, 2, 64, 2>(p, dev, stream, 8, splits);
     case 9: return launch_bf16_tile<192, 256, 2, 2, 64, 2>(p, dev, stream, 9, splits);
-    case 10: return launch_bf16_tile<256, 384, 2, 2, 64, 2, true>(p, dev, stream, 10, splits);
-    case 11: return launch_bf16_tile<384, 192, 2, 2, 64, 2, true>(p, dev, stream, 11, splits);
+    case 10: return launch_bf16_tile<256, 384, 2, 2, 64, 2, 1>(p, dev, stream, 10, splits);
+    case 11: return launch_bf16_tile<384, 192, 2, 2, 64, 2, 1>(p, dev, stream, 11, splits);
+    case 12: return launch_bf16_tile<256, 384, 2, 2, 64, 2, 2>(p, dev, stream, 12, splits);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }

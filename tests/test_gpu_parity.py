@@ -147,7 +147,7 @@ def _run_and_compare(flow, ops, dtype, tol, out_dtype=None):
     return err
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12])
 @pytest.mark.parametrize("flow", ["os", "ls", "rs"])
 def test_bf16_random_cases_all_variants(flow, variant):
     _lib.check(_lib.load().ms_set_variant(variant))
@@ -180,7 +180,7 @@ def test_bf16_output_is_one_rounding_of_the_fp32_accumulator():
     assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 3, 5, 8, 10, 11])
+@pytest.mark.parametrize("variant", [0, 1, 3, 5, 8, 10, 11, 12])
 @pytest.mark.parametrize("flow", ["ls", "rs"])
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
 def test_bf16_chunks_are_one_rounding_of_the_fp32_chunks(flow, variant, in_dtype):
@@ -443,7 +443,7 @@ def test_nan_and_inf_propagate():
 
 
 # ------------------------------------------------------------------ fused output-stationary epilogue
-@pytest.mark.parametrize("variant", [0, 1, 3, 4, 7, 8, 9, 10, 11])
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 7, 8, 9, 10, 11, 12])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_fused_epilogue_gelu_residual_moments(variant, out_dtype):
     """ms_gemm_os_fused: Y = gelu(sum_k A_k B_k) + residual, plus the row sums / sums of squares of Y
