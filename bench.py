@@ -24,10 +24,10 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2516.6     # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
 PEAK_FP32_TFLOPS = 157.3      # MI355X dense fp32 MFMA
 # Bytes per launch of the config-2 kernel that cross the L2 <-> fabric boundary (Infinity Cache or HBM).  This is an
-# OFFLINE figure: two rocprofv3 --pmc runs of this program (FETCH_SIZE 692250 KiB-units x 2.0 and WRITE_SIZE 104960 x 1.0,
+# OFFLINE figure: two rocprofv3 --pmc runs of this program (FETCH_SIZE 698639 KiB-units x 1.9999 and WRITE_SIZE 114688 x 1.0,
 # each scaled by what the same counter reads for a 1 GiB device copy in the same run), valid for the kernel variant
 # named beside it.  It is reported only when the launch this run timed used that variant (ms_query tells).
-TRAFFIC_PROFILE = {"bytes": 1525127376, "variant": 10,
+TRAFFIC_PROFILE = {"bytes": int(round(698639.1 * 1024 * 1048576 / 524313.19 + 114688 * 1024)), "variant": 10,
                    "source": "profiles/gemm_bf16_big_256x384x64_os_cfg2.md @ variant 10 (gemm_bf16_big_kernel<4,6>, 256x384x64 tile)"}
 SETTLE_LAUNCHES = 60          # untimed launches before the warm-up: the package power controller's start-up transient
 
