@@ -233,7 +233,7 @@ def Cannon_LS(X, W, i, j, R, C, K, B):
 
 
 def Cannon_RS(X, W, i, j, R, C, K, B):
-    """reference :302-342."""
+    """reference :379-417 (the definition in force: it shadows the one at :302-342, which computes the same product)."""
     return _ring_rs("cannon", X, W, i, j, R, C)
 
 
@@ -241,21 +241,29 @@ def Cannon_RS(X, W, i, j, R, C, K, B):
 # mesh completion: what psum_scatter + the (.., K, B) interleave do with the partial chunks
 # ------------------------------------------------------------------------------------------------
 
+def _block(extent: int, B: int) -> int:
+    """Largest block size <= B (a power of two) in which ``extent`` divides: the unsliced bodies have no block size of
+    their own, and a window of any width is a whole number of blocks of 1."""
+    while B > 1 and extent % B:
+        B //= 2
+    return max(B, 1)
+
+
 def _finish(chunks_by_peer, me, axis, B, dtype):
     """psum_scatter over the peers (device ``me`` of them keeps its window of every summed chunk) and the
     interleave of the K windows into the output shard: reference :182-193 (LS: peers = the mesh row,
-    axis 1) and :204-214 (RS: peers = the mesh column, axis 0).  One kernel; the sum is fp32 in peer
-    order with one rounding to ``dtype``."""
+    axis 1) and :204-214 (RS: peers = the mesh column, axis 0); with one chunk per peer it is the tiled scatter of
+    the unsliced bodies (:27, :32).  One layout kernel; the sum is fp32 in peer order with one rounding to ``dtype``.
+    More than 64 chunk pointers (P * K) do not fit one launch: the peers are then summed group by group into fp32
+    shards, and one more launch adds those up and rounds."""
     P, K = len(chunks_by_peer), len(chunks_by_peer[0])
-    if P * K > 64:  # more pointers than one launch takes: sum the peers first, then place
-        tot = []
-        for k in range(K):
-            t = chunks_by_peer[0][k].clone()
-            for p in range(1, P):
-                t += chunks_by_peer[p][k]
-            tot.append(t)
-        chunks_by_peer = [tot]
-    return slice_layout.unpack_chunks(chunks_by_peer, B, axis, window=me, parts=P, out_dtype=dtype)
+    if P * K <= 64:
+        return slice_layout.unpack_chunks(chunks_by_peer, B, axis, window=me, parts=P, out_dtype=dtype)
+    g = max(1, 64 // K)
+    partial = [slice_layout.unpack_chunks(chunks_by_peer[p0:p0 + g], B, axis, window=me, parts=P, out_dtype=torch.float32)
+               for p0 in range(0, P, g)]
+    width = partial[0].shape[1] if axis == 1 else partial[0].shape[0]
+    return slice_layout.unpack_chunks([[t] for t in partial], _block(width, 8), axis, window=0, parts=1, out_dtype=dtype)
 
 
 class ShardedMatmul:
@@ -319,19 +327,15 @@ class ShardedMatmul:
             rows = []
             for i in range(R):
                 chunks = [run(i, j) for j in range(C)]
-                if not self.sliced:  # one chunk: tiled scatter of contiguous column blocks
-                    tot = sum(c[0] for c in chunks)
-                    rows.append(tot.to(X.dtype))
-                else:
-                    rows.append(torch.cat([_finish(chunks, j, 1, B, X.dtype) for j in range(C)], dim=1))
+                # (unsliced bodies bring one chunk each: the tiled scatter of contiguous column blocks)
+                Bw = B if self.sliced else _block(chunks[0][0].shape[1] // C, 8)
+                rows.append(torch.cat([_finish(chunks, j, 1, Bw, X.dtype) for j in range(C)], dim=1))
             return torch.cat(rows, dim=0)
         cols = []
         for j in range(C):
             chunks = [run(i, j) for i in range(R)]
-            if not self.sliced:
-                cols.append(sum(c[0] for c in chunks).to(X.dtype))
-            else:
-                cols.append(torch.cat([_finish(chunks, i, 0, B, X.dtype) for i in range(R)], dim=0))
+            Bw = B if self.sliced else _block(chunks[0][0].shape[0] // R, 8)
+            cols.append(torch.cat([_finish(chunks, i, 0, Bw, X.dtype) for i in range(R)], dim=0))
         return torch.cat(cols, dim=1)
 
 

@@ -567,7 +567,8 @@ def literal_cannon_ls(X, W, R, C):
 
 
 def literal_cannon_rs(X, W, R, C):
-    """Cannon_RS (TensorParallel.py:302-342)."""
+    """Cannon_RS (TensorParallel.py:379-417, the definition in force; the earlier one at :302-342 that it shadows
+    issues the same products, shifts and sums in the same order)."""
     assert R == C
     N = C
     Xs, Ws = _shards(X, R, C), _shards(W, R, C)
