@@ -55,6 +55,16 @@ template __global__ void msk::gemm_bf16_x16_kernel<true, true, false, false>(con
 template __global__ void msk::gemm_bf16_x16_kernel<true, true, true, false>(const msk::GemmArgs);
 template __global__ void msk::gemm_bf16_x16_kernel<false, false, false, false>(const msk::GemmArgs);
 template __global__ void msk::gemm_bf16_x16_kernel<false, false, true, false>(const msk::GemmArgs);
+#define MS_INSTANTIATE_F32(WGM, WGN)                                                                          \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, true, false, true>(const msk::GemmArgs);     \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, true, false, false>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, true, true, true>(const msk::GemmArgs);      \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, true, true, false>(const msk::GemmArgs);     \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, false, false, true>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, false, false, false>(const msk::GemmArgs);
+MS_INSTANTIATE_F32(4, 2)
+MS_INSTANTIATE_F32(2, 2)
+#undef MS_INSTANTIATE_F32
 
 namespace {
 thread_local char g_err[512] = "";
@@ -393,8 +403,12 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   return launch_variant(single.v, single.splits, p, dev, stream);
 }
 
-int launch_f32(const Problem &p, hipStream_t stream) {
-  msk::GemmArgsF32 g;
+// fp32 operands: gemm_f32_tile_kernel on 256 x 128 tiles (eight waves), or on 128 x 128 ones (four waves) when the
+// larger tile would leave compute units without work
+template <int WGM, int WGN>
+int launch_f32_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+  constexpr int BM = 64 * WGM, BN = 64 * WGN;
+  msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
   for (int i = 0; i < p.na; i++) g.a[i] = p.a[i];
   for (int i = 0; i < p.nb; i++) g.b[i] = p.b[i];
@@ -404,19 +418,34 @@ int launch_f32(const Problem &p, hipStream_t stream) {
   g.a_by_chunk = p.flow == RS;
   g.b_by_chunk = p.flow == LS;
   g.M = p.M; g.N = p.N; g.K = p.K;
-  if (p.flow == RS) { g.a_rs = 1; g.a_cs = p.lda; } else { g.a_rs = p.lda; g.a_cs = 1; }
-  if (p.flow == LS) { g.b_rs = 1; g.b_cs = p.ldb; } else { g.b_rs = p.ldb; g.b_cs = 1; }
-  g.ldc = p.ldc;
-  g.tiles_m = (p.M + 63) / 64;
-  g.tiles_n = (p.N + 63) / 64;
+  g.lda = p.lda; g.ldb = p.ldb; g.ldc = p.ldc;
+  g.tiles_m = (p.M + BM - 1) / BM;
+  g.tiles_n = (p.N + BN - 1) / BN;
   const long total = (long)g.tiles_m * g.tiles_n * g.nchunks;
   if (total > 0x7FFFFFFF) return fail(MS_ERR_ARG, "problem has too many tiles");
-  dim3 gd((unsigned)total), bd(256);
-  if (p.out_dtype == MS_DTYPE_BF16) hipLaunchKernelGGL(msk::gemm_f32_kernel<true>, gd, bd, 0, stream, g);
-  else hipLaunchKernelGGL(msk::gemm_f32_kernel<false>, gd, bd, 0, stream, g);
+  g.total_tiles = (int)total;
+  g.group_m = 8;
+  g.splits = 1;
+  dim3 gd(dev.cus < total ? dev.cus : (int)total), bd(WGM * WGN * 64);
+  const bool obf = p.out_dtype == MS_DTYPE_BF16;
+  if (p.flow == OS) {
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, true, false, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, true, false, false><<<gd, bd, 0, stream>>>(g);
+  } else if (p.flow == LS) {
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, true, true, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, true, true, false><<<gd, bd, 0, stream>>>(g);
+  } else {
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, false, false, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, false, false, false><<<gd, bd, 0, stream>>>(g);
+  }
   g_launches++;
   MS_HIP(hipGetLastError());
   return MS_OK;
+}
+
+int launch_f32(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+  const long big = (long)((p.M + 255) / 256) * ((p.N + 127) / 128) * (p.flow == OS ? 1 : p.S);
+  return big >= dev.cus ? launch_f32_tile<4, 2>(p, dev, stream) : launch_f32_tile<2, 2>(p, dev, stream);
 }
 
 int run(const Problem &p, void *stream) {
@@ -429,7 +458,7 @@ int run(const Problem &p, void *stream) {
   g_launches = 0;
   g_last_variant = 0;
   g_last_splits = 1;
-  return p.in_dtype == MS_DTYPE_BF16 ? launch_bf16(p, *dev, st) : launch_f32(p, st);
+  return p.in_dtype == MS_DTYPE_BF16 ? launch_bf16(p, *dev, st) : launch_f32(p, *dev, st);
 }
 
 int timed(const Problem &p, void *stream, int warmup, int reps, float *ms_out) {

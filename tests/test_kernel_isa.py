@@ -25,7 +25,7 @@ def gemm_asm(tmp_path_factory):
                            "-o", str(out), os.path.join(CSRC, "ms_gemm.hip")], cwd=CSRC, stderr=subprocess.DEVNULL)
     text = out.read_text()
     kernels = {}
-    for name in re.findall(r"^(_ZN3msk\w*gemm_bf16_\w+):", text, re.M):
+    for name in re.findall(r"^(_ZN3msk\w*gemm_(?:bf16|f32)_\w+):", text, re.M):
         start = text.index(name + ":")
         kernels[name] = text[start:text.index("s_endpgm", start)].split("\n")
     assert len(kernels) >= 80
