@@ -132,7 +132,9 @@ int ms_workspace_init(void *workspace, size_t bytes, void *stream);
  * Replaces the contractions of MeshFlow_LS (TensorParallel.py:181,187); S == 1 is Collective_LS
  * (TensorParallel.py:26).  A is the device's own shard; W_s the s-th all-gathered row slice of the
  * [out,in] weights; Y_s is the partial-output chunk the mesh reduce-scatters over its columns.
- * Chunks are produced in slice order: every tile of Y_s is scheduled before any tile of Y_{s+1}. */
+ * The tile list is chunk-major and the workgroups take tiles in list order, so the chunks tend to complete in slice
+ * order, but a plain call promises nothing before it has ended on its stream; a consumer that wants Y_s earlier uses
+ * ms_gemm_ls_signal. */
 int ms_gemm_ls(const void *A, int lda, const void *const *W_slices, int ldw, int S,
                int m, int n_slice, int k,
                float *const *Y_chunks, int ldy, int in_dtype, void *stream);
@@ -156,6 +158,22 @@ int ms_gemm_ls_ex(const void *A, int lda, const void *const *W_slices, int ldw, 
 int ms_gemm_rs_ex(const void *const *X_slices, int ldx, const void *W, int ldw, int S,
                   int m_slice, int n, int k,
                   void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream);
+
+/* ms_gemm_ls_ex / ms_gemm_rs_ex with completion counters, so that the reduce-scatter of chunk s (the psum_scatter that
+ * follows each einsum in MeshFlow_LS / MeshFlow_RS, TensorParallel.py:182-189, :204-212) can start while the later
+ * chunks are still being computed.  chunk_done points to S unsigned counters in device memory, zero before the call;
+ * the kernel adds 1 to chunk_done[s] after each output tile of Y_s is in memory (system-scope release: whoever reads
+ * the count, from another stream or, through a copy, from the host, then reads the counted tiles).  Y_s is complete
+ * when chunk_done[s] == *tiles_per_chunk, which the call writes (host memory) before it returns.  The counters are
+ * only added to: clear them before the next call. */
+int ms_gemm_ls_signal(const void *A, int lda, const void *const *W_slices, int ldw, int S,
+                      int m, int n_slice, int k,
+                      void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
+                      unsigned *chunk_done, int *tiles_per_chunk, void *stream);
+int ms_gemm_rs_signal(const void *const *X_slices, int ldx, const void *W, int ldw, int S,
+                      int m_slice, int n, int k,
+                      void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
+                      unsigned *chunk_done, int *tiles_per_chunk, void *stream);
 
 /* Timing helpers (replace the wall-clock loop of CostModel.estimateMatmul, reference
  * CostModel.py:74-98): run the same call `warmup` times untimed, then `reps` times, each launch
@@ -241,6 +259,14 @@ int ms_probe_mfma_stream(const void *operands, float *sink, int iters, int warmu
  * (1..12, 0 = the library's choice) and split the contraction `variant / 100` ways (2..8, 0 = the library's choice;
  * a forced split needs a workspace and an output-stationary product).  Unknown ids are rejected with MS_ERR_ARG. */
 int ms_set_variant(int variant);
+
+/* Compute units that the GEMM launches of the calling thread leave free (default 0; returns MS_ERR_ARG outside
+ * [0, 1024]).  The kernels are persistent, one workgroup per compute unit, each holding all of its unit's registers:
+ * nothing else runs on a unit until its workgroup has ended.  A caller that overlaps the chunks' reduce-scatter with
+ * the product (the point of the sliced dataflows, TensorParallel.py:182-189, :204-212) reserves the units that the
+ * collective's kernels need; multiples of 8 keep the workgroup-to-XCD mapping of the tile walk.  No counterpart in
+ * the reference, where XLA schedules both. */
+int ms_set_reserved_cus(int n);
 
 #ifdef __cplusplus
 }

@@ -34,7 +34,7 @@ LIB_PATH = os.path.join(_HERE, "libmeshslice_hip.so")
 
 EXPORTS = (
     "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
-    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_os_ws", "ms_gemm_os_noalloc", "ms_workspace_bytes", "ms_workspace_init", "ms_time_os_ws", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex",
+    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_os_ws", "ms_gemm_os_noalloc", "ms_workspace_bytes", "ms_workspace_init", "ms_time_os_ws", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_gemm_ls_signal", "ms_gemm_rs_signal", "ms_set_reserved_cus",
     "ms_time_os", "ms_time_ls", "ms_time_rs", "ms_time_ls_ex", "ms_time_rs_ex",
     "ms_pack_slices", "ms_unpack_chunks", "ms_probe_mfma_stream", "ms_probe_mfma_stream_ex",
 )
@@ -59,6 +59,8 @@ def _declare(lib):
     lib.ms_query.restype = c_long
     lib.ms_set_variant.argtypes = [c_int]
     lib.ms_set_variant.restype = c_int
+    lib.ms_set_reserved_cus.argtypes = [c_int]
+    lib.ms_set_reserved_cus.restype = c_int
     os_args = [vpp, vpp, c_int, c_int, c_int, c_int, c_int, c_int, c_vp, c_int, c_int, c_int, c_vp]
     ls_args = [c_vp, c_int, vpp, c_int, c_int, c_int, c_int, c_int, vpp, c_int, c_int, c_vp]
     rs_args = [vpp, c_int, c_vp, c_int, c_int, c_int, c_int, c_int, vpp, c_int, c_int, c_vp]
@@ -80,6 +82,9 @@ def _declare(lib):
     lib.ms_gemm_rs.argtypes = rs_args
     lib.ms_gemm_ls_ex.argtypes = ls_args[:-1] + [c_int, c_vp]      # ..., in_dtype, out_dtype, stream
     lib.ms_gemm_rs_ex.argtypes = rs_args[:-1] + [c_int, c_vp]
+    # ..., in_dtype, out_dtype, chunk_done, tiles_per_chunk, stream
+    lib.ms_gemm_ls_signal.argtypes = ls_args[:-1] + [c_int, c_vp, ctypes.POINTER(c_int), c_vp]
+    lib.ms_gemm_rs_signal.argtypes = rs_args[:-1] + [c_int, c_vp, ctypes.POINTER(c_int), c_vp]
     lib.ms_time_os.argtypes = os_args + [c_int, c_int, fp]
     lib.ms_time_ls.argtypes = ls_args + [c_int, c_int, fp]
     lib.ms_time_rs.argtypes = rs_args + [c_int, c_int, fp]
@@ -98,7 +103,7 @@ def _declare(lib):
     lib.ms_probe_mfma_stream_ex.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, fp, ctypes.POINTER(ctypes.c_double), c_vp]
     lib.ms_probe_mfma_stream_ex.restype = c_int
     for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_time_os", "ms_time_ls", "ms_time_rs",
-              "ms_time_ls_ex", "ms_time_rs_ex"):
+              "ms_time_ls_ex", "ms_time_rs_ex", "ms_gemm_ls_signal", "ms_gemm_rs_signal"):
         getattr(lib, n).restype = c_int
 
 

@@ -85,13 +85,17 @@ thread_local int g_splits = 0;    // forced split count of the contraction (0 = 
 thread_local int g_launches = 0;   // kernels launched by the last GEMM call of this thread
 thread_local int g_last_variant = 0;   // bf16 kernel variant of that call's first launch (0: the fp32 kernel)
 thread_local int g_last_splits = 1;    // and the number of ways it split the contraction
+thread_local int g_reserved_cus = 0;   // compute units the GEMM launches of this thread leave free (ms_set_reserved_cus)
+thread_local int g_last_tiles_per_chunk = 0;   // output tiles per chunk (per output, for OS) of that call's last launch
 
 using msi::fail;
 
-struct DevInfo {
+struct DevFacts {
+  int cus = 0, clock_khz = 0, gfx950 = 0, lds = 0;
+};
+struct DevInfo : DevFacts {
   std::once_flag once;
   hipError_t err = hipSuccess;
-  int cus = 0, clock_khz = 0, gfx950 = 0, lds = 0;
 };
 DevInfo g_dev[64];
 
@@ -138,6 +142,8 @@ struct Problem {
   // workspace for split contractions (null / 0: none, the contraction is never split)
   void *ws = nullptr;
   size_t ws_bytes = 0;
+  // LS / RS: per-chunk completion counters (null: none)
+  unsigned *chunk_done = nullptr;
 };
 
 // Layout of a split-contraction workspace: SPLIT_MAX_BANDS arrival counters per output tile, then one fp32 partial tile
@@ -204,11 +210,11 @@ void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
 }
 
 extern const char *const SPLIT_REFUSALS[];
-int split_refused(const Problem &p, const DevInfo &dev, int variant, int splits);
+int split_refused(const Problem &p, const DevFacts &dev, int variant, int splits);
 
 // tile BM x BN, WGM x WGN waves, NS ring stages of BK_ k-elements; contraction split `splits` ways
 template <int BM, int BN, int WGM, int WGN, int BK_, int NS, int KIND = 0>
-int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream, int variant, int splits) {
+int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, int variant, int splits) {
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
   for (int i = 0; i < p.na; i++) g.a[i] = p.a[i];
@@ -227,6 +233,8 @@ int launch_bf16_tile(const Problem &p, const DevInfo &dev, hipStream_t stream, i
   g.total_tiles = (int)total;
   g.group_m = 8;
   g.splits = 1;
+  g.chunk_done = p.chunk_done;
+  g_last_tiles_per_chunk = g.tiles_m * g.tiles_n;
   if (splits > 1) {
     const int why = split_refused(p, dev, variant, splits);
     if (why) return fail(MS_ERR_ARG, "contraction cannot be split %d ways here: %s", splits, SPLIT_REFUSALS[why]);
@@ -299,7 +307,7 @@ const char *const SPLIT_REFUSALS[] = {"", "only output-stationary products split
                                       "products with a fused epilogue are not split"};
 
 // 0 if problem p can run on tile variant v with its contraction split `splits` ways, else an index into SPLIT_REFUSALS
-int split_refused(const Problem &p, const DevInfo &dev, int v, int splits) {
+int split_refused(const Problem &p, const DevFacts &dev, int v, int splits) {
   const int bm = TILE_OF[v].bm, bn = TILE_OF[v].bn;
   if (splits < 2 || splits > SPLIT_MAX) return 7;
   if (v == 1 || v == 4 || v == 12) return 8;     // 256x256 on four waves: see ring_can_split; the 16x16x32 kernel has none
@@ -315,7 +323,7 @@ int split_refused(const Problem &p, const DevInfo &dev, int v, int splits) {
 }
 
 // the tile shape and split count with the lowest estimated cost for the whole problem
-Pick pick_variant(const Problem &p, const DevInfo &dev) {
+Pick pick_variant(const Problem &p, const DevFacts &dev) {
   struct Cand { int v; double eff; };
   // with two m/n-contiguous operands (RS) the hand-scheduled tiles gain less over the 256x256 ring than with a
   // k-contiguous operand, and the 192-wide ring tiles do best on four 32-deep stages
@@ -339,7 +347,7 @@ Pick pick_variant(const Problem &p, const DevInfo &dev) {
   return best;
 }
 
-int launch_variant(int v, int splits, const Problem &p, const DevInfo &dev, hipStream_t stream) {
+int launch_variant(int v, int splits, const Problem &p, const DevFacts &dev, hipStream_t stream) {
   if (g_launches == 0) { g_last_variant = v; g_last_splits = splits; }
   switch (v) {
     case 1: return launch_bf16_tile<256, 256, 2, 2, 64, 2>(p, dev, stream, 1, splits);
@@ -364,7 +372,7 @@ int launch_variant(int v, int splits, const Problem &p, const DevInfo &dev, hipS
 // instead of 768 tiles of 256x192 in three rounds, 0.76 ms).  The second launch costs about a hundredth of a
 // millisecond (launch gap, one more prologue), which the estimate charges as tile area.  LS / RS are not split:
 // their chunks are promised in slice order.
-int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
   if (g_variant != 0) return launch_variant(g_variant, g_splits > 1 ? g_splits : 1, p, dev, stream);
   const Pick single = pick_variant(p, dev);
@@ -406,7 +414,7 @@ int launch_bf16(const Problem &p, const DevInfo &dev, hipStream_t stream) {
 // fp32 operands: gemm_f32_tile_kernel on 256 x 128 tiles (eight waves), or on 128 x 128 ones (four waves) when the
 // larger tile would leave compute units without work
 template <int WGM, int WGN>
-int launch_f32_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   constexpr int BM = 64 * WGM, BN = 64 * WGN;
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
@@ -426,6 +434,8 @@ int launch_f32_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   g.total_tiles = (int)total;
   g.group_m = 8;
   g.splits = 1;
+  g.chunk_done = p.chunk_done;
+  g_last_tiles_per_chunk = g.tiles_m * g.tiles_n;
   dim3 gd(dev.cus < total ? dev.cus : (int)total), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   if (p.flow == OS) {
@@ -443,9 +453,16 @@ int launch_f32_tile(const Problem &p, const DevInfo &dev, hipStream_t stream) {
   return MS_OK;
 }
 
-int launch_f32(const Problem &p, const DevInfo &dev, hipStream_t stream) {
+int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   const long big = (long)((p.M + 255) / 256) * ((p.N + 127) / 128) * (p.flow == OS ? 1 : p.S);
   return big >= dev.cus ? launch_f32_tile<4, 2>(p, dev, stream) : launch_f32_tile<2, 2>(p, dev, stream);
+}
+
+// the device as this thread's launches may use it: without the compute units it has been told to leave free
+DevFacts usable(const DevInfo &dev) {
+  DevFacts f = dev;
+  f.cus = f.cus - g_reserved_cus > 0 ? f.cus - g_reserved_cus : 1;
+  return f;
 }
 
 int run(const Problem &p, void *stream) {
@@ -458,7 +475,10 @@ int run(const Problem &p, void *stream) {
   g_launches = 0;
   g_last_variant = 0;
   g_last_splits = 1;
-  return p.in_dtype == MS_DTYPE_BF16 ? launch_bf16(p, *dev, st) : launch_f32(p, *dev, st);
+  // the kernels are persistent, one workgroup per compute unit: with units reserved they run on the rest, and the
+  // tile choice plans for that many
+  const DevFacts facts = usable(*dev);
+  return p.in_dtype == MS_DTYPE_BF16 ? launch_bf16(p, facts, st) : launch_f32(p, facts, st);
 }
 
 int timed(const Problem &p, void *stream, int warmup, int reps, float *ms_out) {
@@ -535,6 +555,12 @@ MS_API int ms_set_variant(int variant) {
   if (variant < 0 || v > VARIANTS || splits == 1 || splits > SPLIT_MAX) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
   g_variant = v;
   g_splits = splits;
+  return MS_OK;
+}
+
+MS_API int ms_set_reserved_cus(int n) {
+  if (n < 0 || n > 1024) return fail(MS_ERR_ARG, "ms_set_reserved_cus: %d out of range", n);
+  g_reserved_cus = n;
   return MS_OK;
 }
 
@@ -625,7 +651,7 @@ MS_API int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_
     // what the library would do with room to spare decides whether the built-in scratch is enough
     p.ws = reinterpret_cast<void *>(uintptr_t(256));    // stands for "a workspace": only its size is looked at here
     p.ws_bytes = ~size_t(0);
-    const Pick want = g_variant != 0 ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, *dev);
+    const Pick want = g_variant != 0 ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, usable(*dev));
     if (want.splits > 1) {
       const TileShape t = TILE_OF[want.v];
       const size_t tiles = (size_t)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
@@ -669,6 +695,32 @@ MS_API int ms_gemm_rs_ex(const void *const *X_slices, int ldx, const void *W, in
                          void *const *Y_chunks, int ldy, int in_dtype, int out_dtype, void *stream) {
   const void *w1[1] = {W};
   return run(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype, out_dtype), stream);
+}
+
+// the chunk-producing calls with completion counters
+namespace {
+int run_signal(Problem p, unsigned *chunk_done, int *tiles_per_chunk, void *stream, const char *fn) {
+  if (!chunk_done || !tiles_per_chunk) return fail(MS_ERR_ARG, "%s: null chunk_done / tiles_per_chunk", fn);
+  if (reinterpret_cast<uintptr_t>(chunk_done) & 3) return fail(MS_ERR_ARG, "%s: chunk_done must be 4-byte aligned", fn);
+  p.chunk_done = chunk_done;
+  const int rc = run(p, stream);
+  if (rc == MS_OK) *tiles_per_chunk = g_last_tiles_per_chunk;
+  return rc;
+}
+}  // namespace
+
+MS_API int ms_gemm_ls_signal(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
+                             void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
+                             unsigned *chunk_done, int *tiles_per_chunk, void *stream) {
+  const void *a1[1] = {A};
+  return run_signal(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, Y_chunks, ldy, in_dtype, out_dtype), chunk_done, tiles_per_chunk, stream, "ms_gemm_ls_signal");
+}
+
+MS_API int ms_gemm_rs_signal(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
+                             void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
+                             unsigned *chunk_done, int *tiles_per_chunk, void *stream) {
+  const void *w1[1] = {W};
+  return run_signal(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype, out_dtype), chunk_done, tiles_per_chunk, stream, "ms_gemm_rs_signal");
 }
 
 MS_API int ms_time_os(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,

@@ -210,6 +210,40 @@ def gemm_rs(X_slices: Sequence[torch.Tensor], W: torch.Tensor,
     return call.out
 
 
+def _check_counters(chunk_done: torch.Tensor, S: int, device) -> None:
+    if not (isinstance(chunk_done, torch.Tensor) and chunk_done.is_cuda and chunk_done.device == device
+            and chunk_done.dtype == torch.int32 and chunk_done.is_contiguous() and chunk_done.numel() >= S):
+        raise ValueError(f"chunk_done must be a contiguous int32 tensor of at least {S} counters on {device}")
+
+
+def gemm_ls_signal(A: torch.Tensor, W_slices: Sequence[torch.Tensor], chunk_done: torch.Tensor,
+                   out: Optional[List[torch.Tensor]] = None, out_dtype: Optional[torch.dtype] = None):
+    """gemm_ls with per-chunk completion counters (``ms_gemm_ls_signal``): the kernel adds 1 to ``chunk_done[s]``
+    (int32, zero before the call) after each output tile of ``Y_s`` is in memory, so that the reduce-scatter of chunk
+    s (reference TensorParallel.py:182-189) can start before the call has ended.  Returns ``(chunks, tiles_per_chunk)``:
+    ``Y_s`` is complete when ``chunk_done[s] == tiles_per_chunk``."""
+    call = _prepare_ls(A, W_slices, out, out_dtype)
+    _check_counters(chunk_done, len(W_slices), call.device)
+    tiles = ctypes.c_int(0)
+    with torch.cuda.device(call.device):
+        rc = _lib.load().ms_gemm_ls_signal(*call.args, ctypes.c_void_p(chunk_done.data_ptr()), ctypes.byref(tiles), _stream())
+    _lib.check(rc)
+    return call.out, tiles.value
+
+
+def gemm_rs_signal(X_slices: Sequence[torch.Tensor], W: torch.Tensor, chunk_done: torch.Tensor,
+                   out: Optional[List[torch.Tensor]] = None, out_dtype: Optional[torch.dtype] = None):
+    """gemm_rs with per-chunk completion counters (``ms_gemm_rs_signal``, see gemm_ls_signal; reference
+    TensorParallel.py:204-212)."""
+    call = _prepare_rs(X_slices, W, out, out_dtype)
+    _check_counters(chunk_done, len(X_slices), call.device)
+    tiles = ctypes.c_int(0)
+    with torch.cuda.device(call.device):
+        rc = _lib.load().ms_gemm_rs_signal(*call.args, ctypes.c_void_p(chunk_done.data_ptr()), ctypes.byref(tiles), _stream())
+    _lib.check(rc)
+    return call.out, tiles.value
+
+
 def time_call(flow: str, operands, out, warmup: int = 5, reps: int = 20) -> List[float]:
     """Per-launch milliseconds (HIP events on the current stream) of one local contraction.
 
