@@ -102,8 +102,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 1 GiB device copy (scales rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--only-main", action="store_true", help="skip the S=1 / LS / RS side measurements")
-    ap.add_argument("--kernel-only", choices=("os", "ls", "rs"), default=None,
-                    help="profiling runs: launch only the kernel of configuration 2 (os), 3 (ls) or 4 (rs) and print its time")
+    ap.add_argument("--kernel-only", choices=("os", "ls", "rs", "fp32"), default=None,
+                    help="profiling runs: launch only the kernel of configuration 2 (os), 3 (ls) or 4 (rs), or the fp32 kernel "
+                         "on 4096^3, and print its time")
     ap.add_argument("--variant", type=int, default=0, help="profiling runs: force a bf16 kernel variant (ms_set_variant), 0 = library's choice")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -144,6 +145,12 @@ def main():
             Ws = [W[torch.from_numpy(sel_index(12288, 8, 8, k)).cuda(), :].contiguous() for k in range(8)]
             Y = [torch.empty((4096, 1536), dtype=torch.float32, device="cuda") for _ in range(8)]
             run, fl = (lambda: ms.gemm_ls(X, Ws, out=Y)), flops
+        elif args.kernel_only == "fp32":
+            g = torch.Generator(device="cuda").manual_seed(5)
+            A32 = torch.randn((4096, 4096), generator=g, device="cuda")
+            B32 = torch.randn((4096, 4096), generator=g, device="cuda") * 0.02
+            C32 = torch.empty((4096, 4096), dtype=torch.float32, device="cuda")
+            run, fl = (lambda: ms.gemm_os([A32], [B32], out=C32)), 2.0 * 4096 ** 3
         else:
             g = torch.Generator(device="cuda").manual_seed(4)
             X4 = torch.randn((4096, 3072), generator=g, device="cuda").to(torch.bfloat16)
@@ -163,7 +170,8 @@ def main():
         t = e0.elapsed_time(e1) / args.steps
         print(json.dumps({"kernel_only": args.kernel_only, "kernel_variant": int(lib.ms_query(_lib.MS_QUERY_LAST_VARIANT)),
                           "splits": int(lib.ms_query(_lib.MS_QUERY_LAST_SPLITS)), "steps": args.steps, "kernel_ms_mean": round(t, 4),
-                          "tflops": round(fl / t / 1e9, 1), "frac_of_bf16_peak": round(fl / t / 1e9 / PEAK_BF16_TFLOPS, 4)}), flush=True)
+                          "tflops": round(fl / t / 1e9, 1),
+                          "frac_of_peak": round(fl / t / 1e9 / (PEAK_FP32_TFLOPS if args.kernel_only == "fp32" else PEAK_BF16_TFLOPS), 4)}), flush=True)
         return
 
     # ---- settle phase (always, whatever --warmup says): the first launches after an idle period run up to 30 % slow
