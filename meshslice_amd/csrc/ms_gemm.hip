@@ -55,15 +55,16 @@ template __global__ void msk::gemm_bf16_x16_kernel<true, true, false, false>(con
 template __global__ void msk::gemm_bf16_x16_kernel<true, true, true, false>(const msk::GemmArgs);
 template __global__ void msk::gemm_bf16_x16_kernel<false, false, false, false>(const msk::GemmArgs);
 template __global__ void msk::gemm_bf16_x16_kernel<false, false, true, false>(const msk::GemmArgs);
-#define MS_INSTANTIATE_F32(WGM, WGN)                                                                          \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, true, false, true>(const msk::GemmArgs);     \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, true, false, false>(const msk::GemmArgs);    \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, true, true, true>(const msk::GemmArgs);      \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, true, true, false>(const msk::GemmArgs);     \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, false, false, true>(const msk::GemmArgs);    \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, false, false, false>(const msk::GemmArgs);
-MS_INSTANTIATE_F32(4, 2)
-MS_INSTANTIATE_F32(2, 2)
+#define MS_INSTANTIATE_F32(WGM, WGN, T)                                                                          \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, true>(const msk::GemmArgs);     \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, false>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, true, true>(const msk::GemmArgs);      \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, true, false>(const msk::GemmArgs);     \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, true>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, false>(const msk::GemmArgs);
+MS_INSTANTIATE_F32(4, 2, 2)
+MS_INSTANTIATE_F32(2, 2, 2)
+MS_INSTANTIATE_F32(2, 2, 1)
 #undef MS_INSTANTIATE_F32
 
 namespace {
@@ -421,11 +422,11 @@ int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   return launch_variant(single.v, single.splits, p, dev, stream);
 }
 
-// fp32 operands: gemm_f32_tile_kernel on 256 x 128 tiles (eight waves), or on 128 x 128 ones (four waves) when the
-// larger tile would leave compute units without work
-template <int WGM, int WGN>
+// fp32 operands: gemm_f32_tile_kernel on 256 x 128 tiles (eight waves), or on 128 x 128 / 64 x 64 ones (four waves)
+// when the larger tile would leave compute units without work
+template <int WGM, int WGN, int T>
 int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
-  constexpr int BM = 64 * WGM, BN = 64 * WGN;
+  constexpr int BM = 32 * T * WGM, BN = 32 * T * WGN;
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
   for (int i = 0; i < p.na; i++) g.a[i] = p.a[i];
@@ -449,14 +450,14 @@ int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   dim3 gd(dev.cus < total ? dev.cus : (int)total), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   if (p.flow == OS) {
-    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, true, false, true><<<gd, bd, 0, stream>>>(g);
-    else msk::gemm_f32_tile_kernel<WGM, WGN, true, false, false><<<gd, bd, 0, stream>>>(g);
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, false><<<gd, bd, 0, stream>>>(g);
   } else if (p.flow == LS) {
-    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, true, true, true><<<gd, bd, 0, stream>>>(g);
-    else msk::gemm_f32_tile_kernel<WGM, WGN, true, true, false><<<gd, bd, 0, stream>>>(g);
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, T, true, true, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, T, true, true, false><<<gd, bd, 0, stream>>>(g);
   } else {
-    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, false, false, true><<<gd, bd, 0, stream>>>(g);
-    else msk::gemm_f32_tile_kernel<WGM, WGN, false, false, false><<<gd, bd, 0, stream>>>(g);
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, false><<<gd, bd, 0, stream>>>(g);
   }
   g_launches++;
   MS_HIP(hipGetLastError());
@@ -464,8 +465,11 @@ int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
 }
 
 int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
-  const long big = (long)((p.M + 255) / 256) * ((p.N + 127) / 128) * (p.flow == OS ? 1 : p.S);
-  return big >= dev.cus ? launch_f32_tile<4, 2>(p, dev, stream) : launch_f32_tile<2, 2>(p, dev, stream);
+  const long chunks = p.flow == OS ? 1 : p.S;
+  const long big = (long)((p.M + 255) / 256) * ((p.N + 127) / 128) * chunks;
+  const long mid = (long)((p.M + 127) / 128) * ((p.N + 127) / 128) * chunks;
+  if (big >= dev.cus) return launch_f32_tile<4, 2, 2>(p, dev, stream);
+  return 2 * mid >= dev.cus ? launch_f32_tile<2, 2, 2>(p, dev, stream) : launch_f32_tile<2, 2, 1>(p, dev, stream);
 }
 
 // the device as this thread's launches may use it: without the compute units it has been told to leave free
