@@ -93,6 +93,41 @@ def cpu_baseline(A_host, B_host, flops_full):
             ctx.__exit__(None, None, None)
 
 
+def power_run(torch, run, flops, seconds, what, variant):
+    """Runs `run` back to back for `seconds` while a thread samples `amd-smi metric -p -c`; returns the sustained rate and
+    the mean / max of the socket power and of the first graphics clock it printed."""
+    import re
+    import subprocess
+    import threading
+    samples, stop = [], threading.Event()
+
+    def sampler():
+        while not stop.is_set():
+            try:
+                samples.append(subprocess.run(["amd-smi", "metric", "-p", "-c"], capture_output=True, text=True, timeout=10).stdout)
+            except Exception as e:      # no amd-smi, or no permission: reported as zero samples
+                samples.append("")
+            time.sleep(0.1)
+
+    th = threading.Thread(target=sampler)
+    torch.cuda.synchronize()
+    th.start()
+    t0, n = time.perf_counter(), 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(50):
+            run()
+        torch.cuda.synchronize()
+        n += 50
+    dt = time.perf_counter() - t0
+    stop.set()
+    th.join()
+    watts = [float(m.group(1)) for o in samples[1:] for m in [re.search(r"SOCKET_POWER:\s*([0-9.]+)", o)] if m]
+    mhz = [float(m.group(1)) for o in samples[1:] for m in [re.search(r"GFX_0:\s*\n\s*CLK:\s*([0-9.]+)", o)] if m]
+    stat = lambda v: {"n": len(v), "mean": round(sum(v) / len(v), 1), "max": max(v)} if v else {"n": 0}
+    return {"power_run": what, "kernel_variant": variant, "seconds": round(dt, 2), "launches": n, "tflops": round(flops * n / dt / 1e12, 1),
+            "socket_power_w": stat(watts), "gfx_clk_mhz": stat(mhz)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -105,6 +140,10 @@ def main():
     ap.add_argument("--kernel-only", choices=("os", "ls", "rs", "fp32"), default=None,
                     help="profiling runs: launch only the kernel of configuration 2 (os), 3 (ls) or 4 (rs), or the fp32 kernel "
                          "on 4096^3, and print its time")
+    ap.add_argument("--power", type=float, default=0.0, metavar="SECONDS",
+                    help="with --kernel-only: run the kernel back to back for SECONDS while sampling `amd-smi metric -p -c` "
+                         "(socket power, graphics clock) and print their mean / max")
+    ap.add_argument("--ones", action="store_true", help="with --kernel-only os: all-ones operands (the reference's timing operands)")
     ap.add_argument("--variant", type=int, default=0, help="profiling runs: force a bf16 kernel variant (ms_set_variant), 0 = library's choice")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -158,8 +197,15 @@ def main():
             Xs = [X4[:, torch.from_numpy(sel_index(3072, 4, 8, k)).cuda()].contiguous() for k in range(4)]
             Y = [torch.empty((768, 12288), dtype=torch.float32, device="cuda") for _ in range(4)]
             run, fl = (lambda: ms.gemm_rs(Xs, dY, out=Y)), 2.0 * 3072 * 12288 * 4096
+        if args.ones and args.kernel_only == "os":
+            A = [torch.ones_like(a) for a in A]
+            B = [torch.ones_like(b) for b in B]
+            run = lambda: ms.gemm_os(A, B, out=C)
         for _ in range(SETTLE_LAUNCHES + args.warmup):
             run()
+        if args.power > 0:
+            print(json.dumps(power_run(torch, run, fl, args.power, args.kernel_only, int(lib.ms_query(_lib.MS_QUERY_LAST_VARIANT)))), flush=True)
+            return
         e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         e0.record()

@@ -347,12 +347,12 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   }
   // Two refinements measured on products outside the GPT-3 family (4096 x 11008 x 4096, 8192^3, 5120^3,
   // 16384 x 4096 x 1024, ...), where the estimate above cannot tell the kernels of one tile shape apart:
-  // - 256x384: the 16x16x32 kernel is 5-8 % faster than the 32x32x16 one up to a contraction of about 8192 and 3-4 %
-  //   slower at 12288;
+  // - 256x384: the 16x16x32 kernel is 4-8 % faster than the 32x32x16 one (which stays selectable as variant 10 and
+  //   carries the split contraction);
   // - 256x256: eight waves (two per SIMD) beat four by 1-3 %, by 10-15 % on short contractions, where prologue and
   //   write-out weigh most; only LS on long contractions prefers four.
   if (best.splits == 1) {
-    if (best.v == 10 && total_k <= 10240) best.v = 12;
+    if (best.v == 10) best.v = 12;
     if (best.v == 1 && (p.flow != LS || total_k <= 2048)) best.v = 7;
   }
   return best;
@@ -407,7 +407,7 @@ int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
         const int es_in = 2, es_out = p.out_dtype == MS_DTYPE_BF16 ? 2 : 4;
         Problem head = p;
         head.N = (int)n1;
-        int rc = launch_variant(total_k <= 10240 ? 12 : 10, 1, head, dev, stream);   // (see pick_variant)
+        int rc = launch_variant(12, 1, head, dev, stream);   // (see pick_variant)
         if (rc != MS_OK) return rc;
         const void *b2[MS_MAX_SLICES];
         void *c2[1] = {static_cast<char *>(p.c[0]) + n1 * es_out};
