@@ -27,8 +27,14 @@ PEAK_FP32_TFLOPS = 157.3      # MI355X dense fp32 MFMA
 # OFFLINE figure: two rocprofv3 --pmc runs of this program (FETCH_SIZE 698639 KiB-units x 1.9999 and WRITE_SIZE 114688 x 1.0,
 # each scaled by what the same counter reads for a 1 GiB device copy in the same run), valid for the kernel variant
 # named beside it.  It is reported only when the launch this run timed used that variant (ms_query tells).
-TRAFFIC_PROFILE = {"bytes": int(round(698639.1 * 1024 * 1048576 / 524313.19 + 114688 * 1024)), "variant": 10,
-                   "source": "profiles/gemm_bf16_big_256x384x64_os_cfg2.md @ variant 10 (gemm_bf16_big_kernel<4,6>, 256x384x64 tile)"}
+# HBM-side traffic per config-2 launch from rocprofv3 (FETCH_SIZE x the factor a 1 GiB copy gives in the same run + WRITE_SIZE),
+# per kernel variant: a figure measured offline on that kernel, reported only when the run used it
+TRAFFIC_PROFILES = {
+    12: {"bytes": int(round(689940.0 * 1024 * 1048576 / 524310.0 + 98304 * 1024)),
+         "source": "profiles/gemm_bf16_x16_256x384x64_os_cfg2.md @ variant 12 (gemm_bf16_x16_kernel, 256x384x64 tile)"},
+    10: {"bytes": int(round(698639.1 * 1024 * 1048576 / 524313.19 + 114688 * 1024)),
+         "source": "profiles/gemm_bf16_big_256x384x64_os_cfg2.md @ variant 10 (gemm_bf16_big_kernel<4,6>, 256x384x64 tile)"},
+}
 SETTLE_LAUNCHES = 60          # untimed launches before the warm-up: the package power controller's start-up transient
 
 
@@ -247,12 +253,13 @@ def main():
     # launches: these read a little differently from back-to-back launches and are reported for information)
     per_launch = ms.time_call("os", (A, B), C, warmup=2, reps=min(max(args.steps, 10), 100))
     achieved = flops / (k_ms * 1e-3) / 1e12
-    traffic_ok = variant == TRAFFIC_PROFILE["variant"] and launches == 1
+    traffic_ok = variant in TRAFFIC_PROFILES and launches == 1
+    TRAFFIC_PROFILE = TRAFFIC_PROFILES.get(variant, {})
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                 "traffic": TRAFFIC_PROFILE["bytes"] if traffic_ok else None,
                 "traffic_source": TRAFFIC_PROFILE["source"] if traffic_ok else
-                f"none: this run launched variant {variant} ({launches} launch(es)), the profile covers variant {TRAFFIC_PROFILE['variant']}",
+                f"none: this run launched variant {variant} ({launches} launch(es)), the profiles cover variants {sorted(TRAFFIC_PROFILES)} as one launch",
                 "kernel_variant": variant,
                 "kernel_ms_mean": round(k_ms, 4), "kernel_ms_how": f"two HIP events on the launch stream around the {args.steps} timed launches",
                 "kernel_ms_single_launch_mean": round(float(np.mean(per_launch)), 4),
