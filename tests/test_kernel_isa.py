@@ -1,7 +1,7 @@
 """Properties of the generated gfx950 code that the kernels' speed depends on and that the compiler has broken
 before without any wrong result to show for it: every `buffer_load ... lds` must take its descriptor from scalar
 registers (otherwise each load becomes a loop over the distinct descriptor values), and the K loop of every GEMM
-kernel must not touch scratch memory (a reload there waits for all loads in flight).  Compiles the device code of
+kernel must not touch scratch memory (a reload there waits for all loads in flight) nor spill scalar registers to vector lanes.  Compiles the device code of
 ms_gemm.hip to assembly (no GPU needed) and reads it."""
 import os
 import re
@@ -52,7 +52,7 @@ def test_no_load_is_wrapped_in_a_descriptor_loop(gemm_asm):
 
 
 def test_the_k_loops_do_not_touch_scratch_memory(gemm_asm):
-    offenders = []
+    offenders, lane_spills = [], []
     for name, body in gemm_asm.items():
         # the K loop: the innermost loop that holds the MFMAs of at least two K steps
         inner = None
@@ -63,4 +63,8 @@ def test_the_k_loops_do_not_touch_scratch_memory(gemm_asm):
         assert inner is not None, f"no K loop found in {name}"
         if any("scratch_" in x for x in body[inner[0]:inner[1]]):
             offenders.append(name)
+        # scalar registers spilled to vector lanes cost VALU issue slots between the MFMAs
+        if any("v_readlane" in x or "v_writelane" in x for x in body[inner[0]:inner[1]]):
+            lane_spills.append(name)
     assert not offenders, f"scratch traffic inside the K loop of {offenders}"
+    assert not lane_spills, f"scalar registers spilled to vector lanes inside the K loop of {lane_spills}"
