@@ -70,6 +70,14 @@ def test_default_choice_is_close_to_the_best_variant(flow, shape):
     finally:
         lib.ms_set_variant(0)
     best_v = min(range(1, 13), key=lambda v: times[v])
+    if times[0] > SLACK * times[best_v]:
+        # a host hiccup during the default's loops reads like a bad choice: time the two again before judging
+        try:
+            for v in (0, best_v, 0, best_v):
+                assert lib.ms_set_variant(v) == 0
+                times[v] = min(times[v], _sustained(run))
+        finally:
+            lib.ms_set_variant(0)
     assert times[0] <= SLACK * times[best_v], (
         f"default (variant {picked[0]}, {picked[1]} split(s), {picked[2]} launch(es)) {times[0] * 1e6:.0f} us; "
         f"variant {best_v} {times[best_v] * 1e6:.0f} us; all: " + " ".join(f"{v}:{t * 1e6:.0f}" for v, t in times.items()))
