@@ -270,15 +270,18 @@ def per_slice_shapes(B, I, O, dataflow, meshshape, S, passes=("fwd", "bwd_data",
 
 def sweep_compute_term(meshes=((2, 8), (4, 4), (8, 8)), slice_counts=(1, 2, 4, 8, 16),
                        passes=("fwd",), layers=None, repeat: int = 5, verbose: bool = True, fused: bool = False,
-                       operands=None):
+                       operands=None, vendor: bool = False):
     """Measure every per-slice kernel of the sweep on the GPU and fit the compute term.  ``operands`` ('normal' or
     'ones', default CostModel.DEFAULT_OPERANDS) says what the timing operands hold, see CostModel.estimateMatmul.
 
     Returns ``(ComputeTerm, rows)`` where each row is
     ``(mesh, layer, pass, S, M, N, K, layout, seconds_per_slice)``; with ``fused`` a tenth entry holds the
-    seconds of the one fused S-slice call a device really issues."""
+    seconds of the one fused S-slice call a device really issues, and with ``vendor`` (needs ``fused``) an eleventh the
+    seconds of the vendor library's unsliced product of the same work (CostModel.measureVendorUnsliced)."""
+    if vendor and not fused:
+        raise ValueError("vendor=True compares with the fused call: pass fused=True too")
     layers = layers or gpt3_layers()
-    rows, samples, seen, seen_fused = [], [], {}, {}
+    rows, samples, seen, seen_fused, seen_vendor = [], [], {}, {}, {}
     for mesh in meshes:
         for (lname, B, I, O, dataflow) in layers:
             for S in slice_counts:
@@ -296,6 +299,11 @@ def sweep_compute_term(meshes=((2, 8), (4, 4), (8, 8)), slice_counts=(1, 2, 4, 8
                         row = row + (seen_fused[fk],)
                         ftf = 2.0 * M * N * K * S / seen_fused[fk] / 1e12
                         extra = f" | S x slice {S*seen[key]*1e3:.4f} ms, fused {seen_fused[fk]*1e3:.4f} ms {ftf:.0f} TFLOP/s"
+                        if vendor:
+                            if fk not in seen_vendor:
+                                seen_vendor[fk] = CostModel.measureVendorUnsliced(M, N, K, S, layout=layout, repeat=repeat, operands=operands)
+                            row = row + (seen_vendor[fk],)
+                            extra += f", vendor unsliced {seen_vendor[fk]*1e3:.4f} ms"
                     rows.append(row)
                     if verbose:
                         tf = 2.0 * M * N * K / seen[key] / 1e12
@@ -317,11 +325,12 @@ def _main(argv=None):
     ap.add_argument("--fused", action="store_true", help="also time the fused S-slice call of every row")
     ap.add_argument("--operands", default=CostModel.DEFAULT_OPERANDS, choices=CostModel.OPERAND_KINDS,
                     help="timing operands: N(0, 0.02) samples, or all ones as in the reference")
+    ap.add_argument("--vendor", action="store_true", help="with --fused: also time the vendor library's unsliced product of every row")
     ap.add_argument("--out", default=None, help="write the fitted term and the rows as JSON")
     a = ap.parse_args(argv)
     meshes = [tuple(int(v) for v in m.split("x")) for m in a.meshes.split(",")]
     slices = [int(v) for v in a.slices.split(",")]
-    term, rows = sweep_compute_term(meshes, slices, tuple(a.passes.split(",")), repeat=a.repeat, fused=a.fused, operands=a.operands)
+    term, rows = sweep_compute_term(meshes, slices, tuple(a.passes.split(",")), repeat=a.repeat, fused=a.fused, operands=a.operands, vendor=a.vendor)
     for lay in sorted(term.eta):
         print(f"fit {lay}: t0 = {term.t0[lay]*1e6:.1f} us, eta = {term.eta[lay]:.3f} of {term.peak/1e12:.1f} TFLOP/s")
     CostModel.use_compute_term(term)

@@ -204,6 +204,48 @@ def _time_layout(M, N, K, S, layout, dtype, kind, repeat):
     return float(np.mean(ms)) * 1e-3
 
 
+def measureVendorUnsliced(M, N, K, S, layout: str = "nn", input_precision=None, repeat: int = 5,
+                          operands: Optional[str] = None) -> float:
+    """Seconds of the vendor library's ONE unsliced product that does the work of the fused S-slice call
+    (``torch.matmul``, i.e. hipBLASLt / rocBLAS, on contiguous operands in the layout's own storage; bf16 in and out):
+    'nn' [M, S K] x [S K, N], 'nt' [M, K] x [S N, K]^T, 'tn' [K, S M]^T x [K, N].  A yardstick for the sweep's tables,
+    not a dependency: nothing else in the package calls the library.  Timed like ``measureFused`` (same operand kinds,
+    warm-up counts and HIP events around each launch)."""
+    import torch
+    from . import local_gemm
+    if layout not in ("nn", "nt", "tn"):
+        raise ValueError(f"unknown layout {layout!r}")
+    kind = _operand_kind(operands)
+    if not torch.cuda.is_available():
+        raise local_gemm._lib.MeshSliceError("measureVendorUnsliced needs the GPU")
+    dtype = input_precision or torch.bfloat16
+    M, N, K, S = int(M), int(N), int(K), int(S)
+    mk = lambda shape, i: _timing_operand(shape, dtype, kind, 1 + i)
+    if layout == "nn":
+        a, b = mk((M, S * K), 0), mk((S * K, N), 1)
+        run = lambda out: torch.matmul(a, b, out=out)
+        out = torch.empty((M, N), dtype=dtype, device="cuda")
+    elif layout == "nt":
+        a, b = mk((M, K), 0), mk((S * N, K), 1)
+        run = lambda out: torch.matmul(a, b.t(), out=out)
+        out = torch.empty((M, S * N), dtype=dtype, device="cuda")
+    else:
+        a, b = mk((K, S * M), 0), mk((K, N), 1)
+        run = lambda out: torch.matmul(a.t(), b, out=out)
+        out = torch.empty((S * M, N), dtype=dtype, device="cuda")
+    for _ in range(_WARMUP[kind]):
+        run(out)
+    times = []
+    for _ in range(int(repeat)):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        run(out)
+        e1.record()
+        e1.synchronize()
+        times.append(e0.elapsed_time(e1))
+    return float(np.mean(times)) * 1e-3
+
+
 def estimateMatmul(mesh, M, N, K, input_precision=None, layout: str = "nn", repeat: int = 5,
                    operands: Optional[str] = None) -> float:
     """Seconds of one local ``[M,K] x [K,N]`` contraction (reference CostModel.py:74-98).
