@@ -331,7 +331,9 @@ def main():
         A1 = [torch.randn((512, 256), generator=g, device="cuda") for _ in range(4)]
         B1 = [torch.randn((256, 512), generator=g, device="cuda") for _ in range(4)]
         C32 = torch.empty((512, 512), device="cuda")
-        t = _sustained(lambda: ms.gemm_os(A1, B1, out=C32), 200)
+        # (launches this short are bound by the host's call rate, and one stall of the host thread inside a loop reads as
+        # a many times slower kernel: best of three loops)
+        t = min(_sustained(lambda: ms.gemm_os(A1, B1, out=C32), 200) for _ in range(3))
         extra["fp32_config1_ms"] = round(t, 5); extra["fp32_config1_tflops"] = round(2.0 * 512 * 512 * 1024 / t / 1e9, 2)
         A32 = torch.randn((4096, 4096), generator=g, device="cuda"); B32 = torch.randn((4096, 4096), generator=g, device="cuda")
         C32 = torch.empty((4096, 4096), device="cuda")
