@@ -168,6 +168,28 @@ def test_fp32_random_cases(flow):
         _run_and_compare(flow, ops, torch.float32, TOL_F32)
 
 
+@pytest.mark.parametrize("flow", ["os", "ls", "rs"])
+def test_fp32_long_all_positive_contraction_is_summed_in_blocks(flow):
+    """16384 all-positive terms per output: one fp32 accumulator through the whole contraction drifts to about 2e-6 of
+    the result (measured, with the vendor library as well); summed in blocks of 128 terms the kernel stays near 2e-7.
+    The bound sits between the two, so it fails if the blocks are lost, well before the 1e-5 of the other fp32 tests."""
+    m, n, k, S = 320, 264, 16384, 2
+    g = torch.Generator(device="cuda").manual_seed(11)
+    X = torch.rand((m, k), generator=g, device="cuda")
+    W = torch.rand((k, n), generator=g, device="cuda")
+    want = X.double() @ W.double()
+    if flow == "os":
+        got = ms.gemm_os([X[:, :k // 2].contiguous(), X[:, k // 2:].contiguous()], [W[:k // 2].contiguous(), W[k // 2:].contiguous()])
+    elif flow == "ls":
+        Wt = W.t().contiguous()
+        got = torch.cat(ms.gemm_ls(X, [Wt[:n // 2].contiguous(), Wt[n // 2:].contiguous()], out_dtype=torch.float32), dim=1)
+    else:
+        Xt = X.t().contiguous()
+        got = torch.cat(ms.gemm_rs([Xt[:, :m // 2].contiguous(), Xt[:, m // 2:].contiguous()], W, out_dtype=torch.float32), dim=0)
+    err = ((got.double() - want).norm() / want.norm()).item()
+    assert err < 6e-7, err
+
+
 def test_bf16_output_is_one_rounding_of_the_fp32_accumulator():
     """OS accumulates all slices in fp32 and rounds once: the bf16 result equals the round-to-nearest-even
     of the fp32-output result of the same call, bit for bit."""
