@@ -210,6 +210,20 @@ void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
   }
 }
 
+// Workgroups of a persistent bf16 launch over `items` work items on `units` compute units.  More items than units run in
+// rounds; when the last round would be partly filled, the same number of rounds is run on fewer units instead, all rounds
+// full (a multiple of 8, so that the workgroup -> XCD mapping of the kernels holds).  Under these kernels the device
+// sits on its package power limit: units left idle for the whole launch let the others clock higher, units left idle
+// for the last round only do not (measured on 256 units: 384 tiles of 256x384 in 0.717 ms on 192 units against 0.800 ms
+// on 256; 400 tiles of 256x256 in 0.227 against 0.256 ms; about 0.6 of the last round's idle share is lost either way).
+int balanced_grid(long items, int units) {
+  if (items <= units) return (int)items;
+  const long rounds = (items + units - 1) / units;
+  const long even = ((items + rounds - 1) / rounds + 7) / 8 * 8;
+  return even < units ? (int)even : units;
+}
+constexpr double PARTIAL_ROUND_LOSS = 0.6;
+
 extern const char *const SPLIT_REFUSALS[];
 int split_refused(const Problem &p, const DevFacts &dev, int variant, int splits);
 
@@ -244,7 +258,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
     g.ws_tiles = static_cast<char *>(p.ws) + WS_HEADER_BYTES;
   }
   const long items = total * g.splits;
-  int grid = dev.cus < items ? dev.cus : (int)items;
+  const int grid = balanced_grid(items, dev.cus);
   dim3 gd(grid), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   g.act = p.act; g.res = p.res; g.ldr = p.ldr; g.row_sum = p.row_sum; g.row_sumsq = p.row_sumsq;
@@ -276,10 +290,11 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 //  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel<4, 6>)     11: 384x192, 4 waves, 2 x 64 (gemm_bf16_big_kernel<6, 3>)
 //  12: 256x384, 4 waves, 2 x 64 on the 16x16x32 MFMA (gemm_bf16_x16_kernel)
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
-// ceil(work items / CUs) rounds of one item per CU, so the estimate is rounds x tile area / relative tile
-// efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile reaches 1.06
-// with a k-contiguous A and 1.02 without, the 384x192 tile 1.04 and 0.96, 192-wide ring tiles about 0.93,
-// 128x128 tiles about 0.55).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
+// ceil(work items / CUs) rounds of one item per CU (a partly filled last round is charged in part, see
+// balanced_grid), so the estimate is rounds x tile area / relative tile
+// efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile, on the 16x16x32 kernel
+// that every such pick runs on, reaches 1.12 with a k-contiguous A and 1.09 without, the 384x192 tile 1.04 and 0.96,
+// 192-wide ring tiles about 0.93, 128x128 tiles about 0.55).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
 // k-contiguous: whole 128-byte lines per request, half as many barriers as 32-deep stages.
 //
 // An output-stationary product with fewer tiles than compute units may split its contraction (work items = tiles x
@@ -329,7 +344,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   // with two m/n-contiguous operands (RS) the hand-scheduled tiles gain less over the 256x256 ring than with a
   // k-contiguous operand, and the 192-wide ring tiles do best on four 32-deep stages
   const bool rs = p.flow == RS;
-  const Cand cands[] = {{1, 1.0}, {10, rs ? 1.02 : 1.06}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, 0.55}};
+  const Cand cands[] = {{1, 1.0}, {10, rs ? 1.09 : 1.12}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, 0.55}};
   const long chunks = p.flow == OS ? 1 : p.S;
   const double total_k = (double)p.K * p.S;
   Pick best = {0, 1, 0};
@@ -339,9 +354,15 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
     for (int splits : SPLIT_CHOICES) {
       if (g_splits != 0 && splits != g_splits) continue;
       if (splits > 1 && (split_refused(p, dev, c.v, splits) || (g_splits == 0 && total_k / splits < SPLIT_MIN_K))) continue;
-      const long rounds = (tiles * splits + dev.cus - 1) / dev.cus;
+      // rounds the launch is charged: whole ones, or with the last round partly filled (see balanced_grid) its filled
+      // share plus PARTIAL_ROUND_LOSS of the rest
+      const double exact = (double)(tiles * splits) / dev.cus;
+      const double whole = (double)((tiles * splits + dev.cus - 1) / dev.cus);
+      const double rounds = exact <= 1.0 ? 1.0 : exact + PARTIAL_ROUND_LOSS * (whole - exact);
       const double exchange = splits == 1 ? 0.0 : (SPLIT_FIX + (double)splits * p.M * p.N * SPLIT_PER_ELEMENT) / total_k;
-      const double cost = (double)rounds * bm * bn / c.eff / splits + exchange;
+      // (a split 256x384 product stays on the 32x32x16 kernel, which carries the exchange and is about 5 % slower)
+      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.eff;
+      const double cost = rounds * bm * bn / eff / splits + exchange;
       if (best.v == 0 || cost < best.cost) best = {c.v, splits, cost};
     }
   }
@@ -389,7 +410,7 @@ int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   const Pick single = pick_variant(p, dev);
   if (p.flow == OS && single.splits == 1 && g_splits == 0) {
     constexpr int BM = 256, BN = 384;
-    constexpr double EFF = 1.06;
+    constexpr double EFF = 1.12;
     const long tiles_m = (p.M + BM - 1) / BM;
     const long total_k = (long)p.K * p.S;
     // whole rounds of the big tile: the largest count of leading tile columns whose tiles are a multiple of the CUs
