@@ -343,8 +343,11 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   struct Cand { int v; double eff; };
   // with two m/n-contiguous operands (RS) the hand-scheduled tiles gain less over the 256x256 ring than with a
   // k-contiguous operand, and the 192-wide ring tiles do best on four 32-deep stages
+  // (256x256 is listed on four waves and on eight: unsplit they tie and the refinement below decides, but only the
+  // eight-wave kernel can split its contraction: 2048 x 2048 x 16384 in 0.125 ms on 64 tiles x 4 splits, 0.165 ms on
+  // 256 tiles of 128x128)
   const bool rs = p.flow == RS;
-  const Cand cands[] = {{1, 1.0}, {10, rs ? 1.09 : 1.12}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, 0.55}};
+  const Cand cands[] = {{1, 1.0}, {7, 1.0}, {10, rs ? 1.09 : 1.12}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, 0.55}};
   const long chunks = p.flow == OS ? 1 : p.S;
   const double total_k = (double)p.K * p.S;
   Pick best = {0, 1, 0};
