@@ -293,7 +293,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 // ceil(work items / CUs) rounds of one item per CU (a partly filled last round is charged in part, see
 // balanced_grid), so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile, on the 16x16x32 kernel
-// that every such pick runs on, reaches 1.12 with a k-contiguous A and 1.09 without, the 384x192 tile 1.04 and 0.96,
+// that every such pick runs on, reaches 1.12 (OS) / 1.16 (LS) with a k-contiguous A and 1.09 without, the 384x192 tile 1.04 and 0.96,
 // 192-wide ring tiles about 0.93, 128x128 tiles about 0.55).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
 // k-contiguous: whole 128-byte lines per request, half as many barriers as 32-deep stages.
 //
@@ -343,13 +343,13 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   struct Cand { int v; double eff; };
   // with two m/n-contiguous operands (RS) the hand-scheduled tiles gain less over the 256x256 ring than with a
   // k-contiguous operand, and the 192-wide ring tiles do best on four 32-deep stages
-  // (256x256 is listed on four waves and on eight: unsplit they tie and the refinement below decides, but only the
-  // eight-wave kernel can split its contraction: 2048 x 2048 x 16384 in 0.125 ms on 64 tiles x 4 splits, 0.165 ms on
-  // 256 tiles of 128x128)
-  const bool rs = p.flow == RS;
-  const Cand cands[] = {{1, 1.0}, {7, 1.0}, {10, rs ? 1.09 : 1.12}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, 0.55}};
+  // (256x256 runs on eight waves, two per SIMD: 1-3 % faster than four waves, 10-15 % on short contractions, where
+  // prologue and write-out weigh most, and the one of the two that can split its contraction: 2048 x 2048 x 16384 in
+  // 0.125 ms on 64 tiles x 4 splits, 0.165 ms on 256 tiles of 128x128; four waves stay selectable as variant 1)
+  const bool rs = p.flow == RS, ls = p.flow == LS;
+  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.09 : ls ? 1.16 : 1.12}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, 0.55}};
   const long chunks = p.flow == OS ? 1 : p.S;
-  const double total_k = (double)p.K * p.S;
+  const double total_k = p.flow == OS ? (double)p.K * p.S : (double)p.K;
   Pick best = {0, 1, 0};
   for (const Cand &c : cands) {
     const int bm = TILE_OF[c.v].bm, bn = TILE_OF[c.v].bn;
@@ -361,7 +361,9 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
       // share plus PARTIAL_ROUND_LOSS of the rest
       const double exact = (double)(tiles * splits) / dev.cus;
       const double whole = (double)((tiles * splits + dev.cus - 1) / dev.cus);
-      const double rounds = exact <= 1.0 ? 1.0 : exact + PARTIAL_ROUND_LOSS * (whole - exact);
+      // (the 128x128 kernel does not reach the power limit: its units gain no clock from idle neighbours)
+      const double loss = c.v == 3 ? 1.0 : PARTIAL_ROUND_LOSS;
+      const double rounds = exact <= 1.0 ? 1.0 : exact + loss * (whole - exact);
       const double exchange = splits == 1 ? 0.0 : (SPLIT_FIX + (double)splits * p.M * p.N * SPLIT_PER_ELEMENT) / total_k;
       // (a split 256x384 product stays on the 32x32x16 kernel, which carries the exchange and is about 5 % slower)
       const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.eff;
@@ -369,16 +371,9 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
       if (best.v == 0 || cost < best.cost) best = {c.v, splits, cost};
     }
   }
-  // Two refinements measured on products outside the GPT-3 family (4096 x 11008 x 4096, 8192^3, 5120^3,
-  // 16384 x 4096 x 1024, ...), where the estimate above cannot tell the kernels of one tile shape apart:
-  // - 256x384: the 16x16x32 kernel is 4-8 % faster than the 32x32x16 one (which stays selectable as variant 10 and
-  //   carries the split contraction);
-  // - 256x256: eight waves (two per SIMD) beat four by 1-3 %, by 10-15 % on short contractions, where prologue and
-  //   write-out weigh most; only LS on long contractions prefers four.
-  if (best.splits == 1) {
-    if (best.v == 10) best.v = 12;
-    if (best.v == 1 && (p.flow != LS || total_k <= 2048)) best.v = 7;
-  }
+  // An unsplit 256x384 product runs on the 16x16x32 kernel: 4-8 % faster than the 32x32x16 one, which stays selectable
+  // as variant 10 and carries the split contraction.
+  if (best.splits == 1 && best.v == 10) best.v = 12;
   return best;
 }
 
