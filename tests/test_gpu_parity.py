@@ -161,6 +161,25 @@ def test_bf16_random_cases_all_variants(flow, variant):
         assert err < 1e-5
 
 
+@pytest.mark.parametrize("variant", [3, 7, 8, 10, 11, 12])
+@pytest.mark.parametrize("flow", ["os", "rs"])
+def test_more_tiles_than_compute_units_with_a_partly_filled_last_round(flow, variant):
+    """5120 x 5120 outputs are 280 to 1600 tiles, a whole number of rounds for none of the tile shapes on a device of
+    some hundred compute units: such launches run on fewer workgroups, evenly filled, and every tile must still be
+    computed exactly once (an fp32 result far inside the bf16 tolerance says so: a tile done twice would not show, a
+    tile left out would)."""
+    m = n = 5120; k = 64; S = 2
+    _lib.check(_lib.load().ms_set_variant(variant))
+    ops = _rand_case(flow, m if flow == "os" else m // S, n, k, S, seed=variant, dtype=torch.bfloat16)
+    if flow == "os":
+        got = ms.gemm_os([dev(a, torch.bfloat16) for a in ops[0]], [dev(b, torch.bfloat16) for b in ops[1]], out_dtype=torch.float32)
+        err = orc.rel_frobenius(host(got), orc.oracle_os_block(*ops))
+    else:
+        got = ms.gemm_rs([dev(x, torch.bfloat16) for x in ops[0]], dev(ops[1], torch.bfloat16))
+        err = max(orc.rel_frobenius(host(g), w) for g, w in zip(got, orc.oracle_rs_chunks(*ops)))
+    assert err < 1e-5, err
+
+
 @pytest.mark.parametrize("flow", ["os", "ls", "rs"])
 def test_fp32_random_cases(flow):
     for idx, (m, n, k, S) in enumerate(SHAPES + [(200, 136, 100, 3), (68, 60, 20, 2)]):
