@@ -261,8 +261,8 @@ int ms_probe_mfma_stream(const void *operands, float *sink, int iters, int warmu
 int ms_set_variant(int variant);
 
 /* Compute units that the GEMM launches of the calling thread leave free (default 0; returns MS_ERR_ARG outside
- * [0, 1024]).  The kernels are persistent, one workgroup per compute unit, each holding all of its unit's registers:
- * nothing else runs on a unit until its workgroup has ended.  A caller that overlaps the chunks' reduce-scatter with
+ * [0, 1024]).  The kernels are persistent, at most one workgroup per compute unit (fewer when that fills all rounds of
+ * the launch evenly), each holding all of its unit's registers: nothing else runs on a unit until its workgroup has ended.  A caller that overlaps the chunks' reduce-scatter with
  * the product (the point of the sliced dataflows, TensorParallel.py:182-189, :204-212) reserves the units that the
  * collective's kernels need; multiples of 8 keep the workgroup-to-XCD mapping of the tile walk.  No counterpart in
  * the reference, where XLA schedules both. */
