@@ -50,6 +50,8 @@ extern "C" {
 #define MS_QUERY_LAST_SPLITS 7   /* ways in which that launch split the contraction (1: not split) */
 #define MS_QUERY_LAST_VARIANT 6  /* bf16 kernel variant (tile shape, see ms_set_variant) of the first of those launches; 0 for
                                    the fp32 kernel.  Lets a measurement name the kernel it timed. */
+#define MS_QUERY_LAST_GRID 8     /* workgroups of the first of those launches: the compute units it ran on (at most the
+                                   device's, less the reserved ones; fewer when that fills every round of the launch) */
 
 /* Library version, major*10000 + minor*100 + patch. */
 int ms_version(void);

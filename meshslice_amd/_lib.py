@@ -24,6 +24,7 @@ MS_QUERY_MAX_SLICES = 4
 MS_QUERY_LAST_LAUNCHES = 5
 MS_QUERY_LAST_VARIANT = 6
 MS_QUERY_LAST_SPLITS = 7
+MS_QUERY_LAST_GRID = 8
 MS_ACT_NONE = 0
 MS_ACT_GELU = 1
 MS_MFMA_32X32X16 = 0

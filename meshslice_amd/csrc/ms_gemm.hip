@@ -86,6 +86,7 @@ thread_local int g_splits = 0;    // forced split count of the contraction (0 = 
 thread_local int g_launches = 0;   // kernels launched by the last GEMM call of this thread
 thread_local int g_last_variant = 0;   // bf16 kernel variant of that call's first launch (0: the fp32 kernel)
 thread_local int g_last_splits = 1;    // and the number of ways it split the contraction
+thread_local int g_last_grid = 0;      // and its workgroup count
 thread_local int g_reserved_cus = 0;   // compute units the GEMM launches of this thread leave free (ms_set_reserved_cus)
 thread_local int g_last_tiles_per_chunk = 0;   // output tiles per chunk (per output, for OS) of that call's last launch
 
@@ -278,6 +279,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
     if (obf) launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, false, false, true, false>(gd, bd, stream, g);
     else launch_one<KIND, BM, BN, BK_, NS, WGM, WGN, false, false, false, false>(gd, bd, stream, g);
   }
+  if (g_launches == 0) g_last_grid = grid;
   g_launches++;
   MS_HIP(hipGetLastError());
   return MS_OK;
@@ -478,6 +480,7 @@ int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
     if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, true><<<gd, bd, 0, stream>>>(g);
     else msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, false><<<gd, bd, 0, stream>>>(g);
   }
+  if (g_launches == 0) g_last_grid = (int)gd.x;
   g_launches++;
   MS_HIP(hipGetLastError());
   return MS_OK;
@@ -572,6 +575,7 @@ MS_API long ms_query(int what) {
   if (what == MS_QUERY_LAST_LAUNCHES) return g_launches;
   if (what == MS_QUERY_LAST_VARIANT) return g_last_variant;
   if (what == MS_QUERY_LAST_SPLITS) return g_last_splits;
+  if (what == MS_QUERY_LAST_GRID) return g_last_grid;
   DevInfo *d = nullptr;
   if (dev_info(&d) != MS_OK) return -1;
   switch (what) {

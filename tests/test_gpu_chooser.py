@@ -93,3 +93,31 @@ def test_default_choice_is_close_to_the_best_variant(flow, shape):
     else:
         want, got = f64(X[1][:, rows]).T @ f64(W), f64(Y[1][rows])
     assert orc.rel_frobenius(got, want) <= 1e-2
+
+
+def test_a_partly_filled_last_round_becomes_whole_rounds_on_fewer_units():
+    """400 tiles of 256x256 on a device of 256 units are two rounds: the launch uses 200 workgroups (a multiple of 8),
+    not 256 and then 144; the units it reserves come off first; a launch that fits one round uses one workgroup per tile."""
+    lib = _lib.load()
+    cus = int(lib.ms_query(_lib.MS_QUERY_CU_COUNT))
+    A = [_rand((5120, 256), 1, 1.0)]; B = [_rand((256, 5120), 2, 0.02)]
+    C = torch.empty((5120, 5120), dtype=torch.bfloat16, device="cuda")
+
+    def balanced(items, units):
+        if items <= units:
+            return items
+        rounds = -(-items // units)
+        return min(units, -(-(-(-items // rounds)) // 8) * 8)
+
+    try:
+        for variant, tiles in ((7, 400), (12, 20 * 14), (11, 14 * 27), (8, 20 * 27), (3, 1600)):
+            for reserve in (0, 16):
+                assert lib.ms_set_variant(variant) == 0 and lib.ms_set_reserved_cus(reserve) == 0
+                ms.gemm_os(A, B, out=C)
+                assert lib.ms_query(_lib.MS_QUERY_LAST_GRID) == balanced(tiles, cus - reserve), (variant, reserve)
+        assert lib.ms_set_variant(7) == 0 and lib.ms_set_reserved_cus(0) == 0
+        ms.gemm_os([A[0][:1024]], B, out=C[:1024])
+        assert lib.ms_query(_lib.MS_QUERY_LAST_GRID) == min(cus, 4 * 20)
+    finally:
+        lib.ms_set_variant(0); lib.ms_set_reserved_cus(0)
+    torch.cuda.synchronize()
