@@ -151,6 +151,9 @@ def main():
                          "(socket power, graphics clock) and print their mean / max")
     ap.add_argument("--ones", action="store_true", help="with --kernel-only os: all-ones operands (the reference's timing operands)")
     ap.add_argument("--variant", type=int, default=0, help="profiling runs: force a bf16 kernel variant (ms_set_variant), 0 = library's choice")
+    ap.add_argument("--shape", default=None, metavar="M,N,K",
+                    help="with --kernel-only os: one unsliced bf16 product of this shape instead of configuration 2")
+    ap.add_argument("--reserve", type=int, default=0, help="profiling runs: compute units the kernels leave free (ms_set_reserved_cus)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE mesh device's local GEMM on ONE GPU; --gpus > 1 is not part of this build "
@@ -181,10 +184,19 @@ def main():
         del src, dst
     if args.variant:
         _lib.check(lib.ms_set_variant(args.variant))
+    if args.reserve:
+        _lib.check(lib.ms_set_reserved_cus(args.reserve))
 
     if args.kernel_only:
         # one configuration's kernel alone, for the profiler: settle + warm-up + steps back-to-back launches
-        if args.kernel_only == "os":
+        if args.kernel_only == "os" and args.shape:
+            m_, n_, k_ = (int(v) for v in args.shape.split(","))
+            g = torch.Generator(device="cuda").manual_seed(6)
+            Ax = [torch.randn((m_, k_), generator=g, device="cuda").to(torch.bfloat16)]
+            Bx = [(torch.randn((k_, n_), generator=g, device="cuda") * 0.02).to(torch.bfloat16)]
+            Cx = torch.empty((m_, n_), dtype=torch.bfloat16, device="cuda")
+            run, fl = (lambda: ms.gemm_os(Ax, Bx, out=Cx)), 2.0 * m_ * n_ * k_
+        elif args.kernel_only == "os":
             run, fl = (lambda: ms.gemm_os(A, B, out=C)), flops
         elif args.kernel_only == "ls":
             Ws = [W[torch.from_numpy(sel_index(12288, 8, 8, k)).cuda(), :].contiguous() for k in range(8)]
