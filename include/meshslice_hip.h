@@ -264,7 +264,8 @@ int ms_set_variant(int variant);
 
 /* Compute units that the GEMM launches of the calling thread leave free (default 0; returns MS_ERR_ARG outside
  * [0, 1024]).  The kernels are persistent, at most one workgroup per compute unit (fewer when that fills all rounds of
- * the launch evenly), each holding all of its unit's registers: nothing else runs on a unit until its workgroup has ended.  A caller that overlaps the chunks' reduce-scatter with
+ * the launch evenly; two of the 128x128 kernel while nothing is reserved), holding all of the unit's registers: nothing
+ * else runs on a unit until its workgroup has ended.  A caller that overlaps the chunks' reduce-scatter with
  * the product (the point of the sliced dataflows, TensorParallel.py:182-189, :204-212) reserves the units that the
  * collective's kernels need; multiples of 8 keep the workgroup-to-XCD mapping of the tile walk.  No counterpart in
  * the reference, where XLA schedules both. */

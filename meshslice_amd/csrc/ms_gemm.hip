@@ -225,6 +225,12 @@ int balanced_grid(long items, int units) {
 }
 constexpr double PARTIAL_ROUND_LOSS = 0.6;
 
+// Two workgroups of the 128x128 kernel fit one compute unit (64 KB of LDS and at most 220 registers per lane each) and
+// hide each other's barriers and load latencies: 4096^3 on 1024 such tiles 0.165 -> 0.129 ms, 1536 x 4096 x 2048 0.044 ->
+// 0.029 ms.  Every other kernel takes the unit's registers or LDS for itself.  With units reserved the 128x128 kernel
+// goes back to one workgroup per unit: the dispatcher would spread a larger grid over the reserved units as well.
+int workgroups_per_unit(int variant) { return variant == 3 && g_reserved_cus == 0 ? 2 : 1; }
+
 extern const char *const SPLIT_REFUSALS[];
 int split_refused(const Problem &p, const DevFacts &dev, int variant, int splits);
 
@@ -259,7 +265,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
     g.ws_tiles = static_cast<char *>(p.ws) + WS_HEADER_BYTES;
   }
   const long items = total * g.splits;
-  const int grid = balanced_grid(items, dev.cus);
+  const int grid = balanced_grid(items, workgroups_per_unit(variant) * dev.cus);
   dim3 gd(grid), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   g.act = p.act; g.res = p.res; g.ldr = p.ldr; g.row_sum = p.row_sum; g.row_sumsq = p.row_sumsq;
@@ -296,7 +302,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 // balanced_grid), so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile, on the 16x16x32 kernel
 // that every such pick runs on, reaches 1.12 (OS) / 1.16 (LS) with a k-contiguous A and 1.09 without, the 384x192 tile 1.04 and 0.96,
-// 192-wide ring tiles about 0.93, 128x128 tiles about 0.55).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
+// 192-wide ring tiles about 0.93, 128x128 tiles about 0.55, or 0.42 per workgroup with two of them on a unit).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
 // k-contiguous: whole 128-byte lines per request, half as many barriers as 32-deep stages.
 //
 // An output-stationary product with fewer tiles than compute units may split its contraction (work items = tiles x
@@ -349,7 +355,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   // prologue and write-out weigh most, and the one of the two that can split its contraction: 2048 x 2048 x 16384 in
   // 0.125 ms on 64 tiles x 4 splits, 0.165 ms on 256 tiles of 128x128; four waves stay selectable as variant 1)
   const bool rs = p.flow == RS, ls = p.flow == LS;
-  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.09 : ls ? 1.16 : 1.12}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, 0.55}};
+  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.09 : ls ? 1.16 : 1.12}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, workgroups_per_unit(3) == 2 ? 0.42 : 0.55}};
   const long chunks = p.flow == OS ? 1 : p.S;
   const double total_k = p.flow == OS ? (double)p.K * p.S : (double)p.K;
   Pick best = {0, 1, 0};
@@ -361,8 +367,9 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
       if (splits > 1 && (split_refused(p, dev, c.v, splits) || (g_splits == 0 && total_k / splits < SPLIT_MIN_K))) continue;
       // rounds the launch is charged: whole ones, or with the last round partly filled (see balanced_grid) its filled
       // share plus PARTIAL_ROUND_LOSS of the rest
-      const double exact = (double)(tiles * splits) / dev.cus;
-      const double whole = (double)((tiles * splits + dev.cus - 1) / dev.cus);
+      const long slots = (long)dev.cus * (splits == 1 ? workgroups_per_unit(c.v) : 1);     // (a split launch is one item per unit)
+      const double exact = (double)(tiles * splits) / slots;
+      const double whole = (double)((tiles * splits + slots - 1) / slots);
       // (the 128x128 kernel does not reach the power limit: its units gain no clock from idle neighbours)
       const double loss = c.v == 3 ? 1.0 : PARTIAL_ROUND_LOSS;
       const double rounds = exact <= 1.0 ? 1.0 : exact + loss * (whole - exact);
