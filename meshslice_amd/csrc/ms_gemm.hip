@@ -475,7 +475,16 @@ int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   g.splits = 1;
   g.chunk_done = p.chunk_done;
   g_last_tiles_per_chunk = g.tiles_m * g.tiles_n;
-  dim3 gd(dev.cus < total ? dev.cus : (int)total), bd(WGM * WGN * 64);
+  // Two of the four-wave workgroups fit a compute unit (as with the 128x128 bf16 kernel, see workgroups_per_unit), but
+  // here a unit that holds two takes about 1.75 times as long over them as over one (measured: 512 tiles of 64x64 on
+  // 4096 contraction elements 0.134 ms, against 0.150 ms in two rounds of 256): sharing pays when it saves more
+  // rounds than that, otherwise the launch runs one workgroup per unit in evenly filled rounds.
+  int grid = balanced_grid(total, dev.cus);
+  if (WGM * WGN == 4 && g_reserved_cus == 0 && total > dev.cus) {
+    const long alone = (total + dev.cus - 1) / dev.cus, shared = (total + 2L * dev.cus - 1) / (2L * dev.cus);
+    if (1.75 * shared < alone) grid = total <= 2L * dev.cus ? (int)total : balanced_grid(total, 2 * dev.cus);
+  }
+  dim3 gd(grid), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   if (p.flow == OS) {
     if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, true><<<gd, bd, 0, stream>>>(g);
@@ -498,7 +507,7 @@ int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   const long big = (long)((p.M + 255) / 256) * ((p.N + 127) / 128) * chunks;
   const long mid = (long)((p.M + 127) / 128) * ((p.N + 127) / 128) * chunks;
   if (big >= dev.cus) return launch_f32_tile<4, 2, 2>(p, dev, stream);
-  return 2 * mid >= dev.cus ? launch_f32_tile<2, 2, 2>(p, dev, stream) : launch_f32_tile<2, 2, 1>(p, dev, stream);
+  return mid >= dev.cus ? launch_f32_tile<2, 2, 2>(p, dev, stream) : launch_f32_tile<2, 2, 1>(p, dev, stream);
 }
 
 // the device as this thread's launches may use it: without the compute units it has been told to leave free
