@@ -81,8 +81,10 @@ int ms_gemm_os(const void *const *A_slices, const void *const *B_slices, int S,
  * residual add before a layer norm (:178,:184) and that norm's local row moments, which the mesh
  * then sums over its columns (mn_l / sqmn_l, :125-126: divide by n for the means).
  * activation: MS_ACT_NONE or MS_ACT_GELU (tanh form, the default of jax.nn.gelu).  residual: [m,n] in
- * out_dtype with leading dimension ldr, or NULL.  row_sum / row_sumsq: [m] fp32 vectors the caller has
- * zeroed, or NULL; the order of the atomic additions is not fixed, so their last bits can differ from
+ * out_dtype with leading dimension ldr, or NULL; it may be C itself (every element is read before it is
+ * written), which turns one call per slice into the reference's running sum C += A_s @ B_s
+ * (TensorParallel.py:167) for callers that issue each slice's product as its all-gather completes.
+ * row_sum / row_sumsq: [m] fp32 vectors the caller has zeroed, or NULL; the order of the atomic additions is not fixed, so their last bits can differ from
  * run to run. */
 #define MS_ACT_NONE 0
 #define MS_ACT_GELU 1

@@ -515,6 +515,32 @@ def test_fused_epilogue_gelu_residual_moments(variant, out_dtype):
     assert orc.rel_frobenius(host(s1b), host(plain).sum(1)) <= 1e-4
 
 
+@pytest.mark.parametrize("variant", [0, 3, 7, 8, 10, 11, 12])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+def test_one_call_per_slice_accumulating_in_place_through_the_residual(variant, out_dtype):
+    """The output-stationary product slice by slice, as a mesh would issue it when each slice's call waits for that
+    slice's all-gather: call s adds A_s B_s to C in place (residual = out).  With a bf16 C that is the reference's own
+    arithmetic (the running sum is carried in the input dtype, TensorParallel.py:167); with an fp32 C it equals the
+    one-call product up to the order of the fp32 additions."""
+    _lib.check(_lib.load().ms_set_variant(variant))
+    m, n, k, S = 520, 776, 136, 4
+    A, B = _rand_case("os", m, n, k, S, seed=70 + variant, dtype=torch.bfloat16)
+    a = [dev(x, torch.bfloat16) for x in A]; b = [dev(x, torch.bfloat16) for x in B]
+    C = ms.gemm_os(a[:1], b[:1], out_dtype=out_dtype)
+    for s in range(1, S):
+        ms.gemm_os(a[s:s + 1], b[s:s + 1], out=C, residual=C)
+    if out_dtype == torch.float32:
+        assert orc.rel_frobenius(host(C), orc.oracle_os_block(A, B)) <= 1e-5
+    else:
+        # the oracle's statement of the reference's slice loop: every partial product and every sum rounded to bf16 ...
+        want = orc.bf16_round((A[0].astype(np.float64) @ B[0].astype(np.float64)).astype(np.float32))
+        for s in range(1, S):
+            # ... except that here the product of slice s is added in fp32 before the one rounding of the sum
+            want = orc.bf16_round((want.astype(np.float64) + A[s].astype(np.float64) @ B[s].astype(np.float64)).astype(np.float32))
+        assert orc.rel_frobenius(host(C), want.astype(np.float64)) <= 2e-3       # a bf16 tie now and then falls the other way
+        assert orc.rel_frobenius(host(C), orc.oracle_os_block(A, B)) <= TOL_BF16
+
+
 def test_operand_span_of_2gib_is_rejected():
     """32-bit byte offsets inside the kernels: an operand slice of 2 GiB or more is refused, not mis-addressed."""
     lib = _lib.load()
