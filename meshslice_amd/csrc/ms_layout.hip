@@ -136,7 +136,9 @@ MS_API int ms_unpack_chunks(const void *const *chunks, int P, int S, int ld_chun
   }
   a.dst = out;
   a.rows = rows;
-  const int vec = wide ? 8 : 1;
+  // eight elements per thread, or the four of one 16-byte unit when fp32 chunks of one peer are only moved
+  const bool move_f32 = wide && P == 1 && in_dtype == MS_DTYPE_F32 && out_dtype == MS_DTYPE_F32;
+  const int vec = !wide ? 1 : move_f32 ? 4 : 8;
   a.ucols = cols / vec;
   a.ld_src = ld_chunk;
   a.ld_dst = ld_out;
@@ -150,5 +152,6 @@ MS_API int ms_unpack_chunks(const void *const *chunks, int P, int S, int ld_chun
   dim3 g;
   if (int rc = grid_for(rows, a.ucols, tx, &g, fn)) return rc;
   hipStream_t st = (hipStream_t)stream;
+  if (move_f32) return launch_unpack<float, float, 4>(axis, tx, g, st, a);
   return wide ? launch_unpack_typed<8>(in_dtype, out_dtype, axis, tx, g, st, a) : launch_unpack_typed<1>(in_dtype, out_dtype, axis, tx, g, st, a);
 }
