@@ -18,7 +18,13 @@
  *     elements — implied by the reference's block size of 8; other extents are free;
  *   - calls are asynchronous on `stream` (a hipStream_t; NULL = the default stream);
  *   - return 0 on success, MS_ERR_* (< 0) otherwise; ms_last_error() then describes the failure;
- *   - the library allocates no device memory and keeps no state besides a per-thread error text.
+ *   - the library allocates no device memory.  State it keeps: per host thread, the last error text, the forced tile
+ *     variant (ms_set_variant), the reserved compute units (ms_set_reserved_cus) and what ms_query reports of the
+ *     thread's last call; per process, a table of device facts and, for ms_gemm_os_noalloc alone, one fixed scratch
+ *     array per device in the code object with the stream that used it last;
+ *   - calls from several host threads, and calls on several streams, are safe together; the one shared resource is a
+ *     split-contraction workspace (ms_gemm_os_ws: the caller's; ms_gemm_os_noalloc: the built-in array), whose rules
+ *     stand at those entry points.
  */
 #ifndef MESHSLICE_HIP_H
 #define MESHSLICE_HIP_H
@@ -118,9 +124,15 @@ int ms_gemm_os_ws(const void *const *A_slices, const void *const *B_slices, int 
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  The
  * split-contraction workspace is a fixed array inside the library's code object (4096 + 48 MiB per device, held until the
  * process ends); the call allocates and frees nothing.  A product whose exchange of partial tiles would not fit that
- * array is refused with MS_ERR_UNSUPPORTED (the message names the sizes) — use ms_gemm_os_ws there.  All calls on one
- * device share the array: calls that overlap on a device (different streams without an ordering between them, several
- * host threads) race on it and give wrong results; issue them on one stream or order them with events. */
+ * array is refused with MS_ERR_UNSUPPORTED (the message names the sizes) — use ms_gemm_os_ws there.  Only products that
+ * split their contraction touch the array (few output tiles, a long contraction); all such calls on one device share it.
+ * Calls on one stream are ordered by the stream.  A call that arrives on another stream than the array's previous user
+ * first waits for the device to go idle (hipDeviceSynchronize, under a per-device lock held until the call's kernels
+ * are queued), so eager calls from several streams or host threads never meet in the array — at the price of that wait
+ * whenever the stream changes.  What is NOT ordered: a call made while `stream` is being captured launches nothing
+ * now, so replays of such a graph must be kept from overlapping other users of the array by the caller (replay on one
+ * stream, or order with events); and the first call on a device that needs the array looks its address up
+ * (hipGetSymbolAddress), which should happen outside a capture. */
 int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_slices, int S,
                        int m, int n, int k_slice, int lda, int ldb,
                        void *C, int ldc, int in_dtype, int out_dtype, void *stream);

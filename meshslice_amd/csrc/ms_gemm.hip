@@ -625,21 +625,28 @@ static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
 
 namespace {
 struct ScratchAddr {
-  std::once_flag once;
-  hipError_t err = hipSuccess;
-  void *ptr = nullptr;
+  std::mutex lock;
+  void *ptr = nullptr;             // device address of `scratch` on this device, once looked up
+  hipStream_t last_stream = nullptr;
+  bool used = false;               // a call has used the scratch on last_stream
 };
 ScratchAddr g_scratch[64];
 
-// Device address of `scratch` on the calling thread's current device, looked up once per device with that device current.
-int scratch_address(void **out) {
+// The scratch entry of the calling thread's current device; its address is looked up with that device current on the
+// first call that gets an answer (a failed look-up is reported and tried again by the next call).
+int scratch_address(ScratchAddr **entry) {
   int d = 0;
   MS_HIP(hipGetDevice(&d));
   if (d < 0 || d >= 64) return fail(MS_ERR_HIP, "device ordinal %d out of range", d);
   ScratchAddr &sa = g_scratch[d];
-  std::call_once(sa.once, [&sa]() { sa.err = hipGetSymbolAddress(&sa.ptr, HIP_SYMBOL(scratch)); });
-  if (sa.err != hipSuccess || !sa.ptr) return fail(MS_ERR_HIP, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(sa.err));
-  *out = sa.ptr;
+  std::lock_guard<std::mutex> hold(sa.lock);
+  if (!sa.ptr) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return fail(MS_ERR_HIP, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+    sa.ptr = p;
+  }
+  *entry = &sa;
   return MS_OK;
 }
 
@@ -697,32 +704,50 @@ MS_API int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_
   Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
   int rc = validate(p);
   if (rc) return rc;
-  if (in_dtype == MS_DTYPE_BF16) {
-    DevInfo *dev = nullptr;
-    rc = dev_info(&dev);
-    if (rc) return rc;
-    // what the library would do with room to spare decides whether the built-in scratch is enough
-    p.ws = reinterpret_cast<void *>(uintptr_t(256));    // stands for "a workspace": only its size is looked at here
-    p.ws_bytes = ~size_t(0);
-    const Pick want = g_variant != 0 ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, usable(*dev));
-    if (want.splits > 1) {
-      const TileShape t = TILE_OF[want.v];
-      const size_t tiles = (size_t)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
-      const size_t need = WS_HEADER_BYTES + tiles * want.splits * t.bm * t.bn * sizeof(float);
-      if (need > NOALLOC_SCRATCH_BYTES)
-        return fail(MS_ERR_UNSUPPORTED, "ms_gemm_os_noalloc: this product (m=%d n=%d k=%d x %d slices) would exchange %zu bytes of partial "
-                    "tiles, the built-in scratch holds %zu; use ms_gemm_os_ws with a workspace of ms_workspace_bytes()",
-                    m, n, k_slice, S, need, NOALLOC_SCRATCH_BYTES);
-    }
-    void *ptr = nullptr;
-    rc = scratch_address(&ptr);
-    if (rc) return rc;
-    p.ws = ptr;
-    p.ws_bytes = NOALLOC_SCRATCH_BYTES;
-    // the array keeps what the last call left: the counters must start at zero (a fill kernel, so that the call can be captured)
-    hipLaunchKernelGGL(ws_clear_kernel, dim3(WS_COUNTERS / 256), dim3(256), 0, (hipStream_t)stream, static_cast<int *>(ptr), WS_COUNTERS);
-    MS_HIP(hipGetLastError());
+  if (in_dtype != MS_DTYPE_BF16) return run(p, stream);     // the fp32 kernels never split: no scratch
+  DevInfo *dev = nullptr;
+  rc = dev_info(&dev);
+  if (rc) return rc;
+  // what the library would do with room to spare decides whether the built-in scratch is needed, and whether it is enough
+  p.ws = reinterpret_cast<void *>(uintptr_t(256));    // stands for "a workspace": only its size is looked at here
+  p.ws_bytes = ~size_t(0);
+  const Pick want = g_variant != 0 ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, usable(*dev));
+  if (want.splits <= 1) {
+    // an unsplit product exchanges nothing (without a workspace the library makes the same choice: splits are only ever added)
+    p.ws = nullptr;
+    p.ws_bytes = 0;
+    return run(p, stream);
   }
+  const TileShape t = TILE_OF[want.v];
+  const size_t tiles = (size_t)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
+  const size_t need = WS_HEADER_BYTES + tiles * want.splits * t.bm * t.bn * sizeof(float);
+  if (need > NOALLOC_SCRATCH_BYTES)
+    return fail(MS_ERR_UNSUPPORTED, "ms_gemm_os_noalloc: this product (m=%d n=%d k=%d x %d slices) would exchange %zu bytes of partial "
+                "tiles, the built-in scratch holds %zu; use ms_gemm_os_ws with a workspace of ms_workspace_bytes()",
+                m, n, k_slice, S, need, NOALLOC_SCRATCH_BYTES);
+  ScratchAddr *sa = nullptr;
+  rc = scratch_address(&sa);
+  if (rc) return rc;
+  // A product that splits leaves counters and partial tiles in the one array of its device, so two such calls must not
+  // overlap.  Calls on one stream never do.  A call that comes on ANOTHER stream than the array's previous user first
+  // waits for the device to go idle (hipDeviceSynchronize: allocates nothing), and the entry stays locked until this
+  // call's kernels are queued, so eager calls from several streams or host threads cannot meet in the array.  A stream
+  // under capture launches nothing now and cannot be waited for: how replays of such a graph are ordered against the
+  // array's other users is the caller's business.
+  std::lock_guard<std::mutex> hold(sa->lock);
+  hipStream_t st = (hipStream_t)stream;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  MS_HIP(hipStreamIsCapturing(st, &capturing));
+  if (capturing == hipStreamCaptureStatusNone) {
+    if (sa->used && sa->last_stream != st) MS_HIP(hipDeviceSynchronize());
+    sa->last_stream = st;
+    sa->used = true;
+  }
+  p.ws = sa->ptr;
+  p.ws_bytes = NOALLOC_SCRATCH_BYTES;
+  // the array keeps what the last call left: the counters must start at zero (a fill kernel, so that the call can be captured)
+  hipLaunchKernelGGL(ws_clear_kernel, dim3(WS_COUNTERS / 256), dim3(256), 0, st, static_cast<int *>(sa->ptr), WS_COUNTERS);
+  MS_HIP(hipGetLastError());
   return run(p, stream);
 }
 

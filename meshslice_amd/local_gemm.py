@@ -8,6 +8,7 @@ libmeshslice_hip.so.
 from __future__ import annotations
 
 import ctypes
+import threading
 from typing import List, Optional, Sequence
 
 import torch
@@ -45,36 +46,61 @@ def _same(ts: Sequence[torch.Tensor], name: str):
     return s0
 
 
-_workspaces = {}
+_workspaces = {}            # (device index, stream handle) -> uint8 tensor, least recently used first
+_workspaces_lock = threading.Lock()
+_WORKSPACE_CACHE_MAX = 8      # streams per device that keep a workspace of their own (about 100 MB each)
 
 
-def workspace(device) -> torch.Tensor:
-    """The split-contraction workspace of ``device`` (a uint8 tensor of ``ms_workspace_bytes()`` bytes, allocated and
-    prepared with ``ms_workspace_init`` on first use, then kept): ``gemm_os`` hands it to ``ms_gemm_os_ws`` so that
-    products with few output tiles can spread their contraction over the idle compute units.  Calls that use it
-    must not overlap on the device (they share its counters): issue them on one stream, or order them with events."""
+def workspace(device, stream=None) -> torch.Tensor:
+    """The split-contraction workspace of ``(device, stream)`` (a uint8 tensor of ``ms_workspace_bytes()`` bytes,
+    allocated and prepared with ``ms_workspace_init`` on first use, then kept): ``gemm_os`` hands it to
+    ``ms_gemm_os_ws`` so that products with few output tiles can spread their contraction over the idle compute units.
+
+    Calls that share a workspace must not overlap on the device (they share its arrival counters and partial tiles).
+    Work on ONE stream never overlaps, so every stream gets a workspace of its own (``stream`` defaults to the current
+    one): calls issued from several host threads or on several streams cannot meet in one.  At most
+    ``_WORKSPACE_CACHE_MAX`` streams per device keep one; a further stream evicts the least recently used, after
+    waiting for the device to finish what is queued (the evicted stream may still be running a product on it).
+
+    While a ``torch.cuda.graph`` capture is under way on the current stream the workspace is allocated inside the capture
+    (from the graph's own memory pool, so it lives as long as the graph and later captured calls of the same graph
+    reuse it), prepared by a captured fill kernel and not kept here: a graph's replays never share counters with eager
+    calls or with another graph's."""
     device = torch.device(device)
     idx = device.index if device.index is not None else torch.cuda.current_device()
-    ws = _workspaces.get(idx)
-    if ws is None:
-        if torch.cuda.is_current_stream_capturing():
-            raise _lib.MeshSliceError("the workspace of this device does not exist yet and cannot be allocated while a "
-                                      "graph is being captured: call gemm_os (or local_gemm.workspace) once before the capture")
-        lib = _lib.load()
-        with torch.cuda.device(idx):
-            nbytes = int(lib.ms_workspace_bytes())
-            if nbytes <= 0:
-                raise _lib.MeshSliceError("could not size the workspace: " + _lib.last_error())
-            ws = torch.empty(nbytes, dtype=torch.uint8, device=torch.device("cuda", idx))
-            _lib.check(lib.ms_workspace_init(ctypes.c_void_p(ws.data_ptr()), nbytes, _stream()))
-            torch.cuda.current_stream().synchronize()     # later calls may come on any stream
-        _workspaces[idx] = ws
-    return ws
+    if stream is None:
+        stream = torch.cuda.current_stream(idx)
+    key = (idx, int(stream.cuda_stream))
+    capturing = torch.cuda.is_current_stream_capturing()
+    if not capturing:
+        with _workspaces_lock:
+            ws = _workspaces.pop(key, None)
+            if ws is not None:
+                _workspaces[key] = ws      # most recently used last
+                return ws
+    lib = _lib.load()
+    with torch.cuda.device(idx), torch.cuda.stream(stream):
+        nbytes = int(lib.ms_workspace_bytes())
+        if nbytes <= 0:
+            raise _lib.MeshSliceError("could not size the workspace: " + _lib.last_error())
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=torch.device("cuda", idx))
+        _lib.check(lib.ms_workspace_init(ctypes.c_void_p(ws.data_ptr()), nbytes, ctypes.c_void_p(stream.cuda_stream)))
+    if capturing:
+        return ws
+    with _workspaces_lock:
+        have = _workspaces.setdefault(key, ws)      # (another thread on the same stream may have been faster)
+        mine = [k for k in _workspaces if k[0] == idx and k != key]
+        evicted = [_workspaces.pop(k) for k in mine[:max(0, len(mine) + 1 - _WORKSPACE_CACHE_MAX)]]
+    if evicted:
+        torch.cuda.synchronize(idx)     # their streams may still be running products that use them
+        del evicted
+    return have
 
 
 def _ws_args(device):
+    """(pointer, bytes, tensor): the caller keeps the tensor until its call has been issued"""
     ws = workspace(device)
-    return ctypes.c_void_p(ws.data_ptr()), ws.numel()
+    return ctypes.c_void_p(ws.data_ptr()), ws.numel(), ws
 
 
 class _Call:
@@ -167,7 +193,7 @@ def gemm_os(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor],
                     and t.device == out.device):
                 raise ValueError("row moments must be contiguous fp32 GPU vectors of length m on the output's device")
             moments[idx] = ctypes.c_void_p(t.data_ptr())
-    ws_ptr, ws_bytes = _ws_args(call.device)
+    ws_ptr, ws_bytes, _ws_keep = _ws_args(call.device)
     with torch.cuda.device(call.device):
         rc = _lib.load().ms_gemm_os_ws(*call.args,
                                        _lib.MS_ACT_GELU if activation == "gelu" else _lib.MS_ACT_NONE,
@@ -260,7 +286,7 @@ def time_call(flow: str, operands, out, warmup: int = 5, reps: int = 20) -> List
     if flow == "os":
         call = _prepare_os(first, second, out, None)
         ms = (ctypes.c_float * int(reps))()
-        ws_ptr, ws_bytes = _ws_args(call.device)
+        ws_ptr, ws_bytes, _ws_keep = _ws_args(call.device)
         with torch.cuda.device(call.device):
             rc = lib.ms_time_os_ws(*call.args, ws_ptr, ws_bytes, _stream(), int(warmup), int(reps), ms)
         _lib.check(rc)

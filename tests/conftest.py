@@ -10,6 +10,7 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+    config.addinivalue_line("markers", "perf: asserts on wall-clock behaviour (also marked gpu; deselect with -m 'gpu and not perf')")
 
 
 def _gpu_available():

@@ -174,20 +174,16 @@ def test_a_watcher_that_sees_a_chunk_complete_reads_the_finished_chunk(flow):
     ops = _operands(flow, m, n, k, S, torch.bfloat16)
     out = [torch.zeros((m, n), dtype=torch.bfloat16, device="cuda") for _ in range(S)]
     want = _plain(flow, ops, torch.bfloat16)
-    early = []
-    for attempt in range(5):                  # the first call also loads the kernel's code: it may end before the first poll
-        tiles, final, h, copied, bands = _watch_once(flow, ops, out, S, m, n, BAND)
-        assert final == [tiles] * S
-        # counts never decrease and never pass the tile count
-        assert (np.diff(h, axis=0) >= 0).all() and h.max() <= tiles
-        # whatever the watcher copied after seeing a chunk complete is the finished chunk
-        assert len(copied) == S, "400 polls did not outlast the kernel"
-        for s in range(S):
-            assert torch.equal(out[s], want[s])
-            assert torch.equal(bands[s][0], want[s][:BAND].cpu()), f"chunk {s}: first rows read before they were written"
-            assert torch.equal(bands[s][1], want[s][m - BAND:].cpu()), f"chunk {s}: last rows read before they were written"
-        early = sorted(s for s, r in copied.items() if r)
-        print(f"\n{flow}: {len(h)} polls, chunks read while the kernel ran: {early}")
-        if early and len(h) > 2:
-            break
-    assert early, "no chunk was seen complete before the kernel had ended"
+    tiles, final, h, copied, bands = _watch_once(flow, ops, out, S, m, n, BAND)
+    assert final == [tiles] * S
+    # counts never decrease and never pass the tile count
+    assert (np.diff(h, axis=0) >= 0).all() and h.max() <= tiles
+    # whatever the watcher copied after seeing a chunk complete is the finished chunk
+    assert len(copied) == S, "400 polls did not outlast the kernel"
+    for s in range(S):
+        assert torch.equal(out[s], want[s])
+        assert torch.equal(bands[s][0], want[s][:BAND].cpu()), f"chunk {s}: first rows read before they were written"
+        assert torch.equal(bands[s][1], want[s][m - BAND:].cpu()), f"chunk {s}: last rows read before they were written"
+    # (whether any chunk was seen complete while the kernel still ran is a matter of timing: tests/test_zy_gpu_timing.py)
+    early = sorted(s for s, r in copied.items() if r)
+    print(f"\n{flow}: {len(h)} polls, chunks read while the kernel ran: {early}")

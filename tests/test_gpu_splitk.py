@@ -158,3 +158,86 @@ def test_workspace_rules_of_the_c_abi():
     torch.cuda.synchronize()
     got = ms.gemm_os([A], [B])
     assert orc.rel_frobenius(_f64(got), _f64(A) @ _f64(B)) <= TOL_BF16
+
+
+def test_split_products_on_two_streams_and_threads_do_not_share_a_workspace():
+    """Two host threads, each on a stream of its own, run products that DO split (64 tiles for 256 compute units),
+    twenty rounds each, at the same time: every result equals the same product's single-stream result bit for bit and
+    the float64 oracle to tolerance.  (One workspace shared by both streams would let their arrival counters and
+    partial tiles meet.)"""
+    import threading
+    L = _lib.load()
+    cases = []
+    for t in range(2):
+        A = [_rand((2048, 3072), 1.0, 200 + 10 * t + s) for s in range(4)]
+        B = [_rand((3072, 1536), 0.02, 300 + 10 * t + s) for s in range(4)]
+        alone = ms.gemm_os(A, B)
+        assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) > 1
+        rows = np.random.default_rng(t).choice(2048, 32, replace=False)
+        want = sum(_f64(a[rows]) @ _f64(b) for a, b in zip(A, B))
+        assert orc.rel_frobenius(_f64(alone[rows]), want) <= TOL_BF16
+        cases.append((A, B, alone))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    ready = threading.Barrier(2)
+    bad, errors, split_counts = [], [], [None, None]
+
+    def work(t):
+        try:
+            torch.cuda.set_device(0)
+            A, B, alone = cases[t]
+            outs = [torch.empty_like(alone) for _ in range(20)]
+            with torch.cuda.stream(streams[t]):
+                ms.gemm_os(A, B, out=outs[0])          # (this stream's workspace is made here, before the two meet)
+                streams[t].synchronize()
+                ready.wait()
+                for r in range(20):
+                    ms.gemm_os(A, B, out=outs[r])
+                split_counts[t] = int(_lib.load().ms_query(_lib.MS_QUERY_LAST_SPLITS))
+                streams[t].synchronize()
+            bad.extend((t, r) for r in range(20) if not torch.equal(outs[r], alone))
+        except Exception as e:  # pragma: no cover
+            errors.append(e)
+            ready.abort()
+
+    threads = [threading.Thread(target=work, args=(t,)) for t in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    assert split_counts[0] > 1 and split_counts[1] > 1
+    assert not bad, f"(thread, round) whose result differs from the single-stream result: {bad}"
+    w0 = local_gemm.workspace("cuda", streams[0]); w1 = local_gemm.workspace("cuda", streams[1])
+    assert w0.data_ptr() != w1.data_ptr() != local_gemm.workspace("cuda").data_ptr()
+    # the same two products interleaved from ONE host thread on the two streams
+    outs = [[torch.empty_like(cases[t][2]) for _ in range(10)] for t in range(2)]
+    for r in range(10):
+        for t in range(2):
+            with torch.cuda.stream(streams[t]):
+                ms.gemm_os(cases[t][0], cases[t][1], out=outs[t][r])
+    torch.cuda.synchronize()
+    for t in range(2):
+        for r in range(10):
+            assert torch.equal(outs[t][r], cases[t][2]), (t, r)
+
+
+def test_workspace_cache_keeps_a_bounded_number_of_streams():
+    keep = local_gemm._WORKSPACE_CACHE_MAX
+    streams = [torch.cuda.Stream() for _ in range(3)]
+    try:
+        local_gemm._WORKSPACE_CACHE_MAX = 2
+        first = local_gemm.workspace("cuda", streams[0])
+        assert local_gemm.workspace("cuda", streams[0]) is first
+        local_gemm.workspace("cuda", streams[1])
+        local_gemm.workspace("cuda", streams[2])
+        mine = [k for k in local_gemm._workspaces if k[0] == torch.cuda.current_device()]
+        assert len(mine) == 2 and (torch.cuda.current_device(), streams[2].cuda_stream) in mine
+    finally:
+        local_gemm._WORKSPACE_CACHE_MAX = keep
+    A = [_rand((1024, 2048), 1.0, 90)]; B = [_rand((2048, 768), 0.02, 91)]
+    with torch.cuda.stream(streams[0]):
+        got = ms.gemm_os(A, B)
+    torch.cuda.synchronize()
+    assert orc.rel_frobenius(_f64(got), _f64(A[0]) @ _f64(B[0])) <= TOL_BF16

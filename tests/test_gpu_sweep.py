@@ -56,37 +56,69 @@ def test_the_picks_cover_the_shapes_the_sweep_is_known_for():
         assert _shape(mesh, layer, pname, 4)[3] == layout
 
 
-@pytest.mark.parametrize("S", [1, 4, 16])
-@pytest.mark.parametrize("mesh,layer,pname,layout", PICKS, ids=[f"{m[0]}x{m[1]}-{l}-{p}" for m, l, p, _ in PICKS])
-def test_fused_call_of_a_sweep_shape_matches_the_oracle(mesh, layer, pname, layout, S):
-    M, N, K, lay = _shape(mesh, layer, pname, S)
-    assert lay == layout
+def _check_fused_call(mesh, layer, pname, S, nrows=12, ncols=192):
+    """The one fused S-slice call a device issues for (mesh, layer, pass) against float64 numpy products of the same
+    bf16 values on ``nrows`` sampled rows x ``ncols`` sampled columns of the output (of three chunks for LS / RS)."""
+    M, N, K, layout = _shape(mesh, layer, pname, S)
     key = (mesh, layer, pname, S)
     rng = np.random.default_rng(zlib.crc32(repr(key).encode()))
+    rows = torch.from_numpy(np.sort(rng.choice(M, min(M, nrows), replace=False))).cuda()
+    cols = torch.from_numpy(np.sort(rng.choice(N, min(N, ncols), replace=False))).cuda()
     if layout == "nn":      # C = sum_s A_s @ B_s
         A = [_operand((M, K), key, "a", s) for s in range(S)]
         Bm = [_operand((K, N), key, "b", s) for s in range(S)]
         C = ms.gemm_os(A, Bm)
-        rows = rng.choice(M, 12, replace=False)
-        want = sum(_f64(a[rows]) @ _f64(b) for a, b in zip(A, Bm))
-        assert orc.rel_frobenius(_f64(C[rows]), want) <= TOL_BF16
-        if (M, N, K * S) == (4096, 9216, 12288):
-            assert _lib.load().ms_query(_lib.MS_QUERY_LAST_LAUNCHES) == 2
+        want = sum(_f64(a[rows]) @ _f64(b[:, cols]) for a, b in zip(A, Bm))
+        assert orc.rel_frobenius(_f64(C[rows][:, cols]), want) <= TOL_BF16
     elif layout == "nt":    # Y_s = A @ W_s^T
         A = _operand((M, K), key, "a")
         W = [_operand((N, K), key, "w", s) for s in range(S)]
         Y = ms.gemm_ls(A, W)
-        rows = rng.choice(M, 12, replace=False)
         for s in sorted({0, S // 2, S - 1}):
-            assert orc.rel_frobenius(_f64(Y[s][rows]), _f64(A[rows]) @ _f64(W[s]).T) <= TOL_BF16
+            assert orc.rel_frobenius(_f64(Y[s][rows][:, cols]), _f64(A[rows]) @ _f64(W[s][cols]).T) <= TOL_BF16
     else:                   # Y_s = X_s^T @ W
         X = [_operand((K, M), key, "x", s) for s in range(S)]
         W = _operand((K, N), key, "w")
         Y = ms.gemm_rs(X, W)
-        rows = rng.choice(M, 12, replace=False)
-        Wd = _f64(W)
+        Wd = _f64(W[:, cols])
         for s in sorted({0, S // 2, S - 1}):
-            assert orc.rel_frobenius(_f64(Y[s][rows]), _f64(X[s][:, rows]).T @ Wd) <= TOL_BF16
+            assert orc.rel_frobenius(_f64(Y[s][rows][:, cols]), _f64(X[s][:, rows]).T @ Wd) <= TOL_BF16
+    return M, N, K, layout
+
+
+@pytest.mark.parametrize("S", [1, 4, 16])
+@pytest.mark.parametrize("mesh,layer,pname,layout", PICKS, ids=[f"{m[0]}x{m[1]}-{l}-{p}" for m, l, p, _ in PICKS])
+def test_fused_call_of_a_sweep_shape_matches_the_oracle(mesh, layer, pname, layout, S):
+    M, N, K, lay = _check_fused_call(mesh, layer, pname, S, ncols=1 << 30)      # whole sampled rows
+    assert lay == layout
+    if (M, N, K * S) == (4096, 9216, 12288):
+        assert _lib.load().ms_query(_lib.MS_QUERY_LAST_LAUNCHES) == 2
+
+
+# The sweep of BASELINE's configuration 5 row by row: the four forward GEMMs of one GPT-3-like layer (reference
+# BenchTransformer.py:80-93) on the 2x8, 4x4 and 8x8 meshes at every slice count of the sweep (per-slice shapes by
+# reference CostModel.py:249-285): 60 rows; and one backward-data and one backward-weight row per mesh at S = 2 and 8.
+MESHES = [(2, 8), (4, 4), (8, 8)]
+SLICE_COUNTS = [1, 2, 4, 8, 16]
+FORWARD_ROWS = [(mesh, layer, "fwd", S) for mesh in MESHES for layer in ("in_proj", "out_proj", "ff1", "ff2") for S in SLICE_COUNTS]
+BACKWARD_ROWS = [(mesh, layer, pname, S) for mesh, layer, pname in
+                 [((2, 8), "ff1", "bwd_data"), ((2, 8), "ff2", "bwd_weight"), ((4, 4), "ff2", "bwd_data"), ((4, 4), "ff1", "bwd_weight"),
+                  ((8, 8), "in_proj", "bwd_data"), ((8, 8), "ff2", "bwd_weight")] for S in (2, 8)]
+
+
+def test_the_forward_rows_are_the_sixty_of_the_sweep():
+    assert len(FORWARD_ROWS) == 60 and len(set(FORWARD_ROWS)) == 60
+    assert {_shape(m, l, p, S)[3] for m, l, p, S in FORWARD_ROWS} == {"nn", "nt"}
+    assert {_shape(m, l, p, S)[3] for m, l, p, S in BACKWARD_ROWS} == {"nn", "nt", "tn"}
+    assert _shape((4, 4), "ff1", "fwd", 4) == (4096, 12288, 3072, "nn")           # configuration 2
+    assert _shape((4, 4), "ff2", "fwd", 8) == (4096, 1536, 12288, "nt")           # configuration 3
+    assert _shape((4, 4), "ff1", "bwd_weight", 4) == (3072, 12288, 4096, "tn")    # configuration 4's product, all four slices
+
+
+@pytest.mark.parametrize("mesh,layer,pname,S", FORWARD_ROWS + BACKWARD_ROWS,
+                         ids=[f"{m[0]}x{m[1]}-{l}-{p}-S{S}" for m, l, p, S in FORWARD_ROWS + BACKWARD_ROWS])
+def test_every_row_of_the_sweep_matches_the_oracle(mesh, layer, pname, S):
+    _check_fused_call(mesh, layer, pname, S)
 
 
 @pytest.mark.parametrize("layout,shape", [("nn", (4096, 12288, 3072)), ("nt", (4096, 3072, 9216)), ("tn", (3072, 12288, 8192))])

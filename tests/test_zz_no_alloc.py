@@ -1,10 +1,14 @@
-"""The entry point that allocates nothing (``ms_gemm_os_noalloc``) against ``ms_gemm_os_ws`` through the C ABI: two calls
-in a row, the second with a smaller input, bit for bit; an over-sized product is refused with a message."""
+"""The entry point that allocates nothing (``ms_gemm_os_noalloc``) through the C ABI: against ``ms_gemm_os_ws`` bit for
+bit on two calls in a row, the second with a smaller input, and against the float64 oracle (rel-Frobenius <= 1e-2,
+bf16 in / fp32 accumulate); the device's free memory does not move across the calls; calls that alternate between two
+streams, and replays of a captured call, give the same bits; an over-sized product is refused with a message."""
 import ctypes
 
+import numpy as np
 import pytest
 import torch
 
+from oracle import meshslice_oracle as orc
 from meshslice_amd import _lib, local_gemm
 
 pytestmark = pytest.mark.gpu
@@ -25,9 +29,16 @@ def _both(L, A, B, m, n, k, S):
     splits = L.ms_query(_lib.MS_QUERY_LAST_SPLITS)
     got = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
     torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
     _lib.check(L.ms_gemm_os_noalloc(*head(got), None))
     assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == splits
     torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "device memory was allocated or freed during the call"
+    # and against the float64 oracle on sampled rows
+    rows = np.random.default_rng(m + n).choice(m, min(m, 24), replace=False)
+    f64 = lambda t: t.float().cpu().numpy().astype(np.float64)
+    ref = sum(f64(a[rows]) @ f64(b) for a, b in zip(A, B))
+    assert orc.rel_frobenius(f64(got[rows]), ref) <= 1e-2
     return got, want, splits
 
 
@@ -55,6 +66,64 @@ def test_no_alloc_entry_point_matches_the_workspace_entry_point():
     _lib.check(L.ms_gemm_os_noalloc(pa, pb, 1, 256, 256, 128, 128, 256, ctypes.c_void_p(c32.data_ptr()), 256,
                                     _lib.MS_DTYPE_F32, _lib.MS_DTYPE_F32, None))
     assert torch.allclose(c32, a32 @ b32, rtol=1e-4, atol=1e-3)
+
+
+def _noalloc(L, A, B, C, stream):
+    m, k = A[0].shape; n = B[0].shape[1]
+    pa, _ka = _lib.ptr_array([t.data_ptr() for t in A]); pb, _kb = _lib.ptr_array([t.data_ptr() for t in B])
+    _lib.check(L.ms_gemm_os_noalloc(pa, pb, len(A), m, n, k, A[0].stride(0), B[0].stride(0), ctypes.c_void_p(C.data_ptr()), n,
+                                    _lib.MS_DTYPE_BF16, _lib.MS_DTYPE_BF16, ctypes.c_void_p(stream.cuda_stream)))
+
+
+def test_no_alloc_calls_that_alternate_between_two_streams_do_not_meet_in_the_scratch():
+    """Two different split products, issued alternately on two streams with no ordering of the caller's between them:
+    the entry point itself keeps them apart (it waits for the device when the stream changes)."""
+    L = _lib.load()
+    L.ms_set_variant(0)
+    A1 = [_rand((2048, 3072), 1.0, 61 + s) for s in range(4)]; B1 = [_rand((3072, 1536), 0.02, 71 + s) for s in range(4)]
+    A2 = [_rand((1024, 4096), 1.0, 81 + s) for s in range(2)]; B2 = [_rand((4096, 768), 0.02, 91 + s) for s in range(2)]
+    want1 = torch.empty((2048, 1536), dtype=torch.bfloat16, device="cuda"); want2 = torch.empty((1024, 768), dtype=torch.bfloat16, device="cuda")
+    main = torch.cuda.current_stream()
+    _noalloc(L, A1, B1, want1, main); assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) > 1
+    _noalloc(L, A2, B2, want2, main); assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) > 1
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs1 = [torch.empty_like(want1) for _ in range(8)]; outs2 = [torch.empty_like(want2) for _ in range(8)]
+    for r in range(8):
+        _noalloc(L, A1, B1, outs1[r], s1)
+        _noalloc(L, A2, B2, outs2[r], s2)
+    torch.cuda.synchronize()
+    for r in range(8):
+        assert torch.equal(outs1[r], want1) and torch.equal(outs2[r], want2), r
+
+
+def test_no_alloc_call_replays_from_a_hip_graph():
+    """One warm call outside the capture (it looks the scratch's address up), then the call is captured and replayed
+    with eager calls in between: every replay gives the eager bits."""
+    L = _lib.load()
+    L.ms_set_variant(0)
+    A = [_rand((1024, 2048), 1.0, 101 + s) for s in range(2)]; B = [_rand((2048, 1536), 0.02, 111 + s) for s in range(2)]
+    eager = torch.empty((1024, 1536), dtype=torch.bfloat16, device="cuda")
+    out = torch.empty_like(eager)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        _noalloc(L, A, B, eager, side)
+        assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) > 1
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            _noalloc(L, A, B, out, side)
+        for _ in range(3):
+            out.zero_()
+            side.synchronize()
+            graph.replay()
+            side.synchronize()
+            assert torch.equal(out, eager)
+            again = torch.empty_like(eager)
+            _noalloc(L, A, B, again, side)              # eager work between the replays, same stream
+            side.synchronize()
+            assert torch.equal(again, eager)
+    torch.cuda.synchronize()
 
 
 def test_no_alloc_entry_point_refuses_what_its_scratch_cannot_hold():
