@@ -24,13 +24,12 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2516.6     # MI355X dense bf16 MFMA: 256 CU x 2.4 GHz x 4096 FLOP/clk/CU
 PEAK_FP32_TFLOPS = 157.3      # MI355X dense fp32 MFMA
 # Bytes per launch of the config-2 kernel that cross the L2 <-> fabric boundary (Infinity Cache or HBM).  This is an
-# OFFLINE figure: two rocprofv3 --pmc runs of this program (FETCH_SIZE 698639 KiB-units x 1.9999 and WRITE_SIZE 114688 x 1.0,
-# each scaled by what the same counter reads for a 1 GiB device copy in the same run), valid for the kernel variant
-# named beside it.  It is reported only when the launch this run timed used that variant (ms_query tells).
+# OFFLINE figure: two rocprofv3 --pmc runs of this program (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter
+# reads for a 1 GiB device copy in the same run: 2 KiB and 1 KiB per count), valid for the kernel variant named beside it.  It is reported only when the launch this run timed used that variant (ms_query tells).
 # HBM-side traffic per config-2 launch from rocprofv3 (FETCH_SIZE x the factor a 1 GiB copy gives in the same run + WRITE_SIZE),
 # per kernel variant: a figure measured offline on that kernel, reported only when the run used it
 TRAFFIC_PROFILES = {
-    12: {"bytes": int(round(689940.0 * 1024 * 1048576 / 524310.0 + 98304 * 1024)),
+    12: {"bytes": int(round(688387.0 * 1024 * 1048576 / 524314.0 + 98428.2 * 1024)),
          "source": "profiles/gemm_bf16_x16_256x384x64_os_cfg2.md @ variant 12 (gemm_bf16_x16_kernel, 256x384x64 tile)"},
     10: {"bytes": int(round(698639.1 * 1024 * 1048576 / 524313.19 + 114688 * 1024)),
          "source": "profiles/gemm_bf16_big_256x384x64_os_cfg2.md @ variant 10 (gemm_bf16_big_kernel<4,6>, 256x384x64 tile)"},

@@ -271,6 +271,31 @@ int ms_probe_mfma_stream_ex(const void *operands, float *sink, int shape, int wa
 int ms_probe_mfma_stream(const void *operands, float *sink, int iters, int warmup, int reps,
                          float *ms_out, double *flops_per_launch, void *stream);
 
+/* Measurement aid (no counterpart in the reference): the output-stationary 256x384x64 kernel on the 16x16x32 MFMA
+ * (bf16 in, bf16 out; what ms_gemm_os runs on BASELINE's configuration 2) with parts of its K loop left out, timed on
+ * the caller's operands: what a part costs is the difference to skip = 0 on the same data, tile loop and clock.
+ * skip (one of the built combinations 0, 1, 2, 3, 4, 8, 16, 24) is a sum of
+ *   1  no global -> LDS loads inside the K loop (the stage buffers keep the tile's first two stages),
+ *   2  no fragment reads inside the K loop (the registers keep the tile's first fragments),
+ *   4  no MFMAs (nor, with nothing left to consume them, fragment reads): the operand stream alone,
+ *   8  no wait for the loads before a K step's barrier,   16  no barrier inside the K loop.
+ * With skip != 0 the contents of C are WRONG (and with 8 or 16 the kernel races on its own LDS buffers): C is scratch
+ * here.  Arguments as ms_gemm_os with in_dtype = out_dtype = MS_DTYPE_BF16; launches warmup + reps kernels on `stream`,
+ * waits, and returns the mean milliseconds per launch in *ms_out. */
+int ms_probe_os_parts(int skip, const void *const *A_slices, const void *const *B_slices, int S,
+                      int m, int n, int k_slice, int lda, int ldb, void *C, int ldc,
+                      int warmup, int reps, float *ms_out, void *stream);
+
+/* Measurement aid (no counterpart in the reference): the rate of a bare L2 -> LDS stream.  One workgroup of four
+ * waves per compute unit issues nothing but 128-bit direct-to-LDS buffer loads, 80 KB per workgroup and step (the
+ * stage size of the 256x384x64 kernels); the workgroups that share an XCD walk the same region of region_steps x 80 KB
+ * of `buffer` round and round (8 regions, one per XCD: buffer_bytes >= 8 x region_steps x 81920), so with
+ * region_steps <= 48 every load after the first round hits in that XCD's 4 MB L2.  A wave has at most
+ * in_flight_steps (1..3) steps' loads outstanding.  sink: one float the kernel may write (it never does for finite
+ * data).  Returns the mean milliseconds per launch in *ms_out and the bytes one launch moves in *bytes_per_launch. */
+int ms_probe_l2_lds_stream(const void *buffer, size_t buffer_bytes, int region_steps, int in_flight_steps, int steps,
+                           int warmup, int reps, float *sink, float *ms_out, double *bytes_per_launch, void *stream);
+
 /* Hook for tests and measurements (thread-local): later bf16 calls on this thread use tile variant `variant % 100`
  * (1..12, 0 = the library's choice) and split the contraction `variant / 100` ways (2..8, 0 = the library's choice;
  * a forced split needs a workspace and an output-stationary product).  Unknown ids are rejected with MS_ERR_ARG. */

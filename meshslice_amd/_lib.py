@@ -38,6 +38,7 @@ EXPORTS = (
     "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_os_ws", "ms_gemm_os_noalloc", "ms_workspace_bytes", "ms_workspace_init", "ms_time_os_ws", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_gemm_ls_signal", "ms_gemm_rs_signal", "ms_set_reserved_cus",
     "ms_time_os", "ms_time_ls", "ms_time_rs", "ms_time_ls_ex", "ms_time_rs_ex",
     "ms_pack_slices", "ms_unpack_chunks", "ms_probe_mfma_stream", "ms_probe_mfma_stream_ex",
+    "ms_probe_os_parts", "ms_probe_l2_lds_stream",
 )
 
 _lock = threading.Lock()
@@ -103,6 +104,12 @@ def _declare(lib):
     # operands, sink, shape, waves_per_simd, iters, warmup, reps, ms_out, flops_per_launch, stream
     lib.ms_probe_mfma_stream_ex.argtypes = [c_vp, c_vp, c_int, c_int, c_int, c_int, c_int, fp, ctypes.POINTER(ctypes.c_double), c_vp]
     lib.ms_probe_mfma_stream_ex.restype = c_int
+    # skip, A_slices, B_slices, S, m, n, k_slice, lda, ldb, C, ldc, warmup, reps, ms_out, stream
+    lib.ms_probe_os_parts.argtypes = [c_int, vpp, vpp, c_int, c_int, c_int, c_int, c_int, c_int, c_vp, c_int, c_int, c_int, fp, c_vp]
+    lib.ms_probe_os_parts.restype = c_int
+    # buffer, buffer_bytes, region_steps, in_flight_steps, steps, warmup, reps, sink, ms_out, bytes_per_launch, stream
+    lib.ms_probe_l2_lds_stream.argtypes = [c_vp, ctypes.c_size_t, c_int, c_int, c_int, c_int, c_int, c_vp, fp, ctypes.POINTER(ctypes.c_double), c_vp]
+    lib.ms_probe_l2_lds_stream.restype = c_int
     for n in ("ms_gemm_os", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_time_os", "ms_time_ls", "ms_time_rs",
               "ms_time_ls_ex", "ms_time_rs_ex", "ms_gemm_ls_signal", "ms_gemm_rs_signal"):
         getattr(lib, n).restype = c_int

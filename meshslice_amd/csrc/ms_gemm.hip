@@ -211,18 +211,7 @@ void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
   }
 }
 
-// Workgroups of a persistent bf16 launch over `items` work items on `units` compute units.  More items than units run in
-// rounds; when the last round would be partly filled, the same number of rounds is run on fewer units instead, all rounds
-// full (a multiple of 8, so that the workgroup -> XCD mapping of the kernels holds).  Under these kernels the device
-// sits on its package power limit: units left idle for the whole launch let the others clock higher, units left idle
-// for the last round only do not (measured on 256 units: 384 tiles of 256x384 in 0.717 ms on 192 units against 0.800 ms
-// on 256; 400 tiles of 256x256 in 0.227 against 0.256 ms; about 0.6 of the last round's idle share is lost either way).
-int balanced_grid(long items, int units) {
-  if (items <= units) return (int)items;
-  const long rounds = (items + units - 1) / units;
-  const long even = ((items + rounds - 1) / rounds + 7) / 8 * 8;
-  return even < units ? (int)even : units;
-}
+using msi::balanced_grid;
 constexpr double PARTIAL_ROUND_LOSS = 0.6;
 
 // Two workgroups of the 128x128 kernel fit one compute unit (64 KB of LDS and at most 220 registers per lane each) and
