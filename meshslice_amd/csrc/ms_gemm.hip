@@ -290,7 +290,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 // ceil(work items / CUs) rounds of one item per CU (a partly filled last round is charged in part, see
 // balanced_grid), so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile, on the 16x16x32 kernel
-// that every such pick runs on, reaches 1.12 (OS) / 1.16 (LS) with a k-contiguous A and 1.09 without, the 384x192 tile 1.04 and 0.96,
+// that every such pick runs on, reaches 1.15 (OS) / 1.20 (LS) with a k-contiguous A and 1.13 without, the 384x192 tile 1.04 and 0.96,
 // 192-wide ring tiles about 0.93, 128x128 tiles about 0.55, or 0.42 per workgroup with two of them on a unit).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
 // k-contiguous: whole 128-byte lines per request, half as many barriers as 32-deep stages.
 //
@@ -344,7 +344,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   // prologue and write-out weigh most, and the one of the two that can split its contraction: 2048 x 2048 x 16384 in
   // 0.125 ms on 64 tiles x 4 splits, 0.165 ms on 256 tiles of 128x128; four waves stay selectable as variant 1)
   const bool rs = p.flow == RS, ls = p.flow == LS;
-  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.09 : ls ? 1.16 : 1.12}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, workgroups_per_unit(3) == 2 ? 0.42 : 0.55}};
+  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.13 : ls ? 1.20 : 1.15}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, workgroups_per_unit(3) == 2 ? 0.42 : 0.55}};
   const long chunks = p.flow == OS ? 1 : p.S;
   const double total_k = p.flow == OS ? (double)p.K * p.S : (double)p.K;
   Pick best = {0, 1, 0};
@@ -406,7 +406,7 @@ int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   const Pick single = pick_variant(p, dev);
   if (p.flow == OS && single.splits == 1 && g_splits == 0) {
     constexpr int BM = 256, BN = 384;
-    constexpr double EFF = 1.12;
+    constexpr double EFF = 1.15;
     const long tiles_m = (p.M + BM - 1) / BM;
     const long total_k = (long)p.K * p.S;
     // whole rounds of the big tile: the largest count of leading tile columns whose tiles are a multiple of the CUs
