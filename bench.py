@@ -34,7 +34,7 @@ TRAFFIC_PROFILES = {
     10: {"bytes": int(round(698639.1 * 1024 * 1048576 / 524313.19 + 114688 * 1024)),
          "source": "profiles/gemm_bf16_big_256x384x64_os_cfg2.md @ variant 10 (gemm_bf16_big_kernel<4,6>, 256x384x64 tile)"},
 }
-X16_VARIANTS = (12,)          # bf16 kernel variants that issue v_mfma_f32_16x16x32_bf16 (the others: 32x32x16)
+X16_VARIANTS = (12, 13)         # bf16 kernel variants that issue v_mfma_f32_16x16x32_bf16 (the others: 32x32x16)
 SETTLE_LAUNCHES = 60          # untimed launches before the warm-up: the package power controller's start-up transient
 
 

@@ -47,14 +47,18 @@ MS_INSTANTIATE_RING(192, 256, 64, 2, 2, 2)
 MS_INSTANTIATE_BIG(4, 6)
 MS_INSTANTIATE_BIG(6, 3)
 #undef MS_INSTANTIATE_BIG
-template __global__ void msk::gemm_bf16_x16_kernel<true, false, true, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_x16_kernel<true, false, false, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_x16_kernel<true, false, true, true>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_x16_kernel<true, false, false, true>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_x16_kernel<true, true, false, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_x16_kernel<true, true, true, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_x16_kernel<false, false, false, false>(const msk::GemmArgs);
-template __global__ void msk::gemm_bf16_x16_kernel<false, false, true, false>(const msk::GemmArgs);
+#define MS_INSTANTIATE_X16(BN)                                                                                  \
+  template __global__ void msk::gemm_bf16_x16_kernel<true, false, true, false, 0, BN>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_bf16_x16_kernel<true, false, false, false, 0, BN>(const msk::GemmArgs);   \
+  template __global__ void msk::gemm_bf16_x16_kernel<true, false, true, true, 0, BN>(const msk::GemmArgs);     \
+  template __global__ void msk::gemm_bf16_x16_kernel<true, false, false, true, 0, BN>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_bf16_x16_kernel<true, true, false, false, 0, BN>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_bf16_x16_kernel<true, true, true, false, 0, BN>(const msk::GemmArgs);     \
+  template __global__ void msk::gemm_bf16_x16_kernel<false, false, false, false, 0, BN>(const msk::GemmArgs);  \
+  template __global__ void msk::gemm_bf16_x16_kernel<false, false, true, false, 0, BN>(const msk::GemmArgs);
+MS_INSTANTIATE_X16(384)
+MS_INSTANTIATE_X16(256)
+#undef MS_INSTANTIATE_X16
 #define MS_INSTANTIATE_F32(WGM, WGN, T)                                                                          \
   template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, true>(const msk::GemmArgs);     \
   template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, false>(const msk::GemmArgs);    \
@@ -197,7 +201,7 @@ int validate(const Problem &p) {
 }
 
 // KIND 0: gemm_bf16_ring_kernel<BM, BN, ...>; 1: gemm_bf16_big_kernel (32x32x16 MFMA, 2x2 waves, two 64-deep stages);
-// 2: gemm_bf16_x16_kernel (256x384x64 on the 16x16x32 MFMA)
+// 2: gemm_bf16_x16_kernel (256x384x64 or 256x256x64 on the 16x16x32 MFMA)
 template <int KIND, int BM, int BN, int BK_, int NS, int WGM, int WGN, bool AK, bool BKM, bool OBF, bool EPI>
 void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
   if constexpr (KIND == 0) {
@@ -206,8 +210,8 @@ void launch_one(dim3 gd, dim3 bd, hipStream_t stream, const msk::GemmArgs &g) {
     static_assert(BM % 64 == 0 && BN % 64 == 0 && BK_ == 64 && NS == 2 && WGM == 2 && WGN == 2, "the big-tile kernels are 2 x 2 waves on two 64-deep stages");
     msk::gemm_bf16_big_kernel<BM / 64, BN / 64, AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
   } else {
-    static_assert(BM == 256 && BN == 384 && BK_ == 64 && NS == 2 && WGM == 2 && WGN == 2, "the 16x16x32 kernel has one shape");
-    msk::gemm_bf16_x16_kernel<AK, BKM, OBF, EPI><<<gd, bd, 0, stream>>>(g);
+    static_assert(BM == 256 && (BN == 384 || BN == 256) && BK_ == 64 && NS == 2 && WGM == 2 && WGN == 2, "the 16x16x32 kernel has two shapes");
+    msk::gemm_bf16_x16_kernel<AK, BKM, OBF, EPI, 0, BN><<<gd, bd, 0, stream>>>(g);
   }
 }
 
@@ -285,7 +289,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 //   4: 256x256, 4 waves, 4 x 32     5: 256x192, 4 waves, 4 x 32     6: 192x256, 4 waves, 4 x 32
 //   7: 256x256, 8 waves, 2 x 64     8: 256x192, 4 waves, 2 x 64     9: 192x256, 4 waves, 2 x 64
 //  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel<4, 6>)     11: 384x192, 4 waves, 2 x 64 (gemm_bf16_big_kernel<6, 3>)
-//  12: 256x384, 4 waves, 2 x 64 on the 16x16x32 MFMA (gemm_bf16_x16_kernel)
+//  12: 256x384, 4 waves, 2 x 64 on the 16x16x32 MFMA (gemm_bf16_x16_kernel)     13: 256x256, the same kernel
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
 // ceil(work items / CUs) rounds of one item per CU (a partly filled last round is charged in part, see
 // balanced_grid), so the estimate is rounds x tile area / relative tile
@@ -302,11 +306,12 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 // 2048 x 1536 x 12288 (64 tiles of 256x192): 170 us unsplit, 100 / 85 / 88 us with 2 / 3 / 4 splits.
 struct Pick { int v, splits; double cost; };
 
-constexpr int VARIANTS = 12;
+constexpr int VARIANTS = 13;
 struct TileShape { int bm, bn; };
 constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256}, {128, 128}, {256, 256}, {256, 192},
                                              {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192},
-                                             {256, 384}};
+                                             {256, 384}, {256, 256}};
+constexpr double X16_OVER_RING_256 = 1.10;   // unsplit 256x256: the 16x16x32 kernel (variant 13) against the eight-wave ring kernel (variant 7)
 constexpr int SPLIT_CHOICES[] = {1, 2, 3, 4, 6, 8};
 constexpr int SPLIT_MAX = 8;
 constexpr long SPLIT_MIN_K = 512;            // contraction elements per split item, at least
@@ -323,7 +328,7 @@ const char *const SPLIT_REFUSALS[] = {"", "only output-stationary products split
 int split_refused(const Problem &p, const DevFacts &dev, int v, int splits) {
   const int bm = TILE_OF[v].bm, bn = TILE_OF[v].bn;
   if (splits < 2 || splits > SPLIT_MAX) return 7;
-  if (v == 1 || v == 4 || v == 12) return 8;     // 256x256 on four waves: see ring_can_split; the 16x16x32 kernel has none
+  if (v == 1 || v == 4 || v == 12 || v == 13) return 8;     // 256x256 on four waves: see ring_can_split; the 16x16x32 kernels have none
   if (p.act || p.res || p.row_sum || p.row_sumsq) return 9;   // see ring_can_split, big_can_split
   if (p.flow != OS) return 1;
   if (!p.ws) return 2;
@@ -363,8 +368,9 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
       const double loss = c.v == 3 ? 1.0 : PARTIAL_ROUND_LOSS;
       const double rounds = exact <= 1.0 ? 1.0 : exact + loss * (whole - exact);
       const double exchange = splits == 1 ? 0.0 : (SPLIT_FIX + (double)splits * p.M * p.N * SPLIT_PER_ELEMENT) / total_k;
-      // (a split 256x384 product stays on the 32x32x16 kernel, which carries the exchange and is about 5 % slower)
-      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.eff;
+      // (a split 256x384 product stays on the 32x32x16 kernel, which carries the exchange and is about 5 % slower; an
+      // unsplit 256x256 one runs on the 16x16x32 kernel, 7-14 % faster than the eight-wave ring kernel that carries the split)
+      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * X16_OVER_RING_256 : c.eff;
       const double cost = rounds * bm * bn / eff / splits + exchange;
       if (best.v == 0 || cost < best.cost) best = {c.v, splits, cost};
     }
@@ -372,6 +378,9 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   // An unsplit 256x384 product runs on the 16x16x32 kernel: 4-8 % faster than the 32x32x16 one, which stays selectable
   // as variant 10 and carries the split contraction.
   if (best.splits == 1 && best.v == 10) best.v = 12;
+  // Likewise an unsplit 256x256 product (4096^3 in 0.093-0.095 ms against 0.106 ms on the ring kernel, 4096 x 4096 x 14336 in
+  // 0.302-0.309 against 0.344 ms); the eight-wave ring kernel stays selectable as variant 7 and carries the split contraction.
+  if (best.splits == 1 && best.v == 7) best.v = 13;
   return best;
 }
 
@@ -390,6 +399,7 @@ int launch_variant(int v, int splits, const Problem &p, const DevFacts &dev, hip
     case 10: return launch_bf16_tile<256, 384, 2, 2, 64, 2, 1>(p, dev, stream, 10, splits);
     case 11: return launch_bf16_tile<384, 192, 2, 2, 64, 2, 1>(p, dev, stream, 11, splits);
     case 12: return launch_bf16_tile<256, 384, 2, 2, 64, 2, 2>(p, dev, stream, 12, splits);
+    case 13: return launch_bf16_tile<256, 256, 2, 2, 64, 2, 2>(p, dev, stream, 13, splits);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }

@@ -56,7 +56,7 @@ def test_default_choice_is_right_on_products_outside_the_gpt3_family(flow, shape
     assert lib.ms_set_variant(0) == 0
     run, check = operands(flow, shape)
     run()
-    assert 1 <= lib.ms_query(_lib.MS_QUERY_LAST_VARIANT) <= 12
+    assert 1 <= lib.ms_query(_lib.MS_QUERY_LAST_VARIANT) <= 13
     assert check() <= 1e-2
 
 
@@ -75,7 +75,7 @@ def test_a_partly_filled_last_round_becomes_whole_rounds_on_fewer_units():
         return min(units, -(-(-(-items // rounds)) // 8) * 8)
 
     try:
-        for variant, tiles in ((7, 400), (12, 20 * 14), (11, 14 * 27), (8, 20 * 27), (3, 1600)):
+        for variant, tiles in ((7, 400), (13, 400), (12, 20 * 14), (11, 14 * 27), (8, 20 * 27), (3, 1600)):
             for reserve in (0, 16):
                 assert lib.ms_set_variant(variant) == 0 and lib.ms_set_reserved_cus(reserve) == 0
                 ms.gemm_os(A, B, out=C)
