@@ -377,32 +377,13 @@ def main():
         t = min(_sustained(lambda: ms.gemm_os(A1, B1, out=C32), 200) for _ in range(3))
         extra["fp32_config1_ms"] = round(t, 5); extra["fp32_config1_tflops"] = round(2.0 * 512 * 512 * 1024 / t / 1e9, 2)
         del A1, B1, C32
-        # fused epilogue: GELU folded into the config-2 product vs the product followed by a separate GELU kernel
-        def _events(f, n):
-            for _ in range(3):
-                f()
-            torch.cuda.synchronize()
-            ts = []
-            for _ in range(n):
-                e0 = torch.cuda.Event(enable_timing=True); e1 = torch.cuda.Event(enable_timing=True)
-                e0.record(); f(); e1.record(); torch.cuda.synchronize()
-                ts.append(e0.elapsed_time(e1))
-            return median(ts)
-        extra["os_s4_fused_gelu_ms"] = round(_events(lambda: ms.gemm_os(A, B, out=C, activation="gelu"), 10), 4)
-        extra["os_s4_then_separate_gelu_ms"] = round(_events(
-            lambda: torch.nn.functional.gelu(ms.gemm_os(A, B, out=C), approximate="tanh"), 10), 4)
-        # the vendor library's GEMM (hipBLASLt through torch.matmul) on the same un-sliced operands, same box, for scale
-        torch.matmul(X, W)
-        extra["vendor_library_matmul_s1_ms"] = round(_events(lambda: torch.matmul(X, W), 30), 4)
-        extra["os_s1_same_method_ms"] = round(_events(lambda: ms.gemm_os([X], [W], out=C), 30), 4)
-        # the layout kernels either side of the GEMM on the same [4096, 12288] bf16 shard: algorithmic GB/s (HBM roofline 8000)
-        from meshslice_amd.slice_layout import measure_rates
-        for label, t, nbytes in measure_rates(dtypes=(torch.bfloat16,), reduce_case=False, reps=24):
-            key = "layout_" + label.replace("bfloat16 ", "").replace(" of the shard", "").replace("=", "").replace(" ", "_").lower() + "_gbps"
-            extra[key] = round(nbytes / t / 1e9, 0)
-        # one device's whole output-stationary step on a 4x4 mesh: cut its own X shard [4096, 3072] and W shard [3072, 12288]
-        # into the S slices it sends to its peers (the peers' slices arrive by all-gather), then the sliced GEMM
-        from meshslice_amd.slice_layout import pack_slices
+        # fused epilogue: GELU folded into the config-2 product vs the product followed by a separate GELU kernel; the vendor
+        # library's GEMM (hipBLASLt through torch.matmul) on the same un-sliced operands, same box, for scale; and one device's
+        # whole output-stationary step on a 4x4 mesh: cut its own X shard [4096, 3072] and W shard [3072, 12288] into the S
+        # slices it sends to its peers (the peers' slices arrive by all-gather), then the sliced GEMM.  All measured like the
+        # other legs: launches back to back between two HIP events after a settle phase (a launch timed alone, the device
+        # idling before it, reads 3-15 % longer and says little about a training step).
+        from meshslice_amd.slice_layout import measure_rates, pack_slices
         Xown, Wown = X[:, :K // 4].contiguous(), W[:K // 4, :].contiguous()
         xs = pack_slices(Xown, S, 8, 1); ws = pack_slices(Wown, S, 8, 0)
 
@@ -410,8 +391,20 @@ def main():
             pack_slices(Xown, S, 8, 1, out=xs)
             pack_slices(Wown, S, 8, 0, out=ws)
             ms.gemm_os(A, B, out=C)
-        extra["os_s4_device_step_ms"] = round(_events(_device_step, 20), 4)
-        extra["os_s4_gemm_alone_same_method_ms"] = round(_events(lambda: ms.gemm_os(A, B, out=C), 20), 4)
+        torch.matmul(X, W)
+        t_plain, t_gelu, t_sep, t_vendor, t_step = _legs([
+            lambda: ms.gemm_os(A, B, out=C), lambda: ms.gemm_os(A, B, out=C, activation="gelu"),
+            lambda: torch.nn.functional.gelu(ms.gemm_os(A, B, out=C), approximate="tanh"),
+            lambda: torch.matmul(X, W), _device_step])
+        extra["os_s4_fused_gelu_ms"] = round(t_gelu, 4)
+        extra["os_s4_then_separate_gelu_ms"] = round(t_sep, 4)
+        extra["vendor_library_matmul_s1_ms"] = round(t_vendor, 4)
+        extra["os_s4_device_step_ms"] = round(t_step, 4)
+        extra["os_s4_gemm_alone_same_method_ms"] = round(t_plain, 4)
+        # the layout kernels either side of the GEMM on the same [4096, 12288] bf16 shard: algorithmic GB/s (HBM roofline 8000)
+        for label, t, nbytes in measure_rates(dtypes=(torch.bfloat16,), reduce_case=False, reps=24):
+            key = "layout_" + label.replace("bfloat16 ", "").replace(" of the shard", "").replace("=", "").replace(" ", "_").lower() + "_gbps"
+            extra[key] = round(nbytes / t / 1e9, 0)
         # what this device sustains on a bare stream of one MFMA instruction (no memory traffic) for operands drawn
         # like X: the practical, power-limited ceiling beside the data-sheet peak.  Both bf16 shapes are measured; the
         # ceiling the timed kernel is held against is that of the instruction it issues (variant 12: 16x16x32).
