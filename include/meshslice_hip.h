@@ -191,6 +191,30 @@ int ms_gemm_rs_signal(const void *const *X_slices, int ldx, const void *W, int l
                       void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
                       unsigned *chunk_done, int *tiles_per_chunk, void *stream);
 
+/* ms_gemm_os_ws (without the fused epilogue) whose kernel reads slice s of A and of B only after slice_ready[s] has
+ * become non-zero: the output-stationary body of the reference gathers slice k + 1 while slice k is being multiplied
+ * (MeshFlow_OS, TensorParallel.py:163-171, where XLA overlaps the all-gathers with the einsum of the slice before);
+ * here the product is ONE launch that may be enqueued before any slice has arrived, and whoever fills slice s (a
+ * gather on another stream) sets slice_ready[s] afterwards, with ms_signal_set on that stream or with any store that
+ * is a release at system scope.  slice_ready points to S + 1 words of device memory: words 0 .. S-1 are the flags,
+ * zero until their slice is complete (flags of slices that are already there are set before the call); word S must be
+ * zero before the call and is set to 1 by the kernel when a wait for a slice lasted longer than timeout_ms (1..60000):
+ * the kernel then goes on and ends, and the contents of C are void.  The caller reads that word after the stream has
+ * been synchronised.
+ * The kernels are persistent and hold every register of the compute units they run on (see ms_set_reserved_cus): a
+ * producer that needs compute units of this device (a copy or collective kernel) only runs beside a waiting product if
+ * units have been reserved for it; without them both stand still until the timeout. */
+int ms_gemm_os_gated(const void *const *A_slices, const void *const *B_slices, int S,
+                     int m, int n, int k_slice, int lda, int ldb,
+                     void *C, int ldc, int in_dtype, int out_dtype,
+                     void *workspace, size_t workspace_bytes,
+                     unsigned *slice_ready, unsigned timeout_ms, void *stream);
+
+/* Sets *flag = value (device memory) once everything enqueued on `stream` before the call has completed, as a release
+ * at system scope: the producer's half of ms_gemm_os_gated (and a way to clear or preset flags in stream order).  No
+ * counterpart in the reference, where XLA orders the gathers and the einsums. */
+int ms_signal_set(unsigned *flag, unsigned value, void *stream);
+
 /* Timing helpers (replace the wall-clock loop of CostModel.estimateMatmul, reference
  * CostModel.py:74-98): run the same call `warmup` times untimed, then `reps` times, each launch
  * bracketed by HIP events on `stream`; ms_out[r] receives the r-th launch's milliseconds.

@@ -150,6 +150,9 @@ struct Problem {
   size_t ws_bytes = 0;
   // LS / RS: per-chunk completion counters (null: none)
   unsigned *chunk_done = nullptr;
+  // OS: per-slice input gate (null: none) and the longest wait for one slice, in ticks of the 100 MHz wall clock
+  unsigned *slice_ready = nullptr;
+  unsigned long long gate_ticks = 0;
 };
 
 // Layout of a split-contraction workspace: SPLIT_MAX_BANDS arrival counters per output tile, then one fp32 partial tile
@@ -249,6 +252,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
   g.group_m = 8;
   g.splits = 1;
   g.chunk_done = p.chunk_done;
+  g.slice_ready = p.slice_ready; g.gate_ticks = p.gate_ticks;
   g_last_tiles_per_chunk = g.tiles_m * g.tiles_n;
   if (splits > 1) {
     const int why = split_refused(p, dev, variant, splits);
@@ -385,6 +389,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
 }
 
 int launch_variant(int v, int splits, const Problem &p, const DevFacts &dev, hipStream_t stream) {
+  if (p.slice_ready && (v == 1 || v == 4)) return fail(MS_ERR_UNSUPPORTED, "tile variant %d has no input gate (256x256 on four waves of the ring kernel)", v);
   if (g_launches == 0) { g_last_variant = v; g_last_splits = splits; }
   switch (v) {
     case 1: return launch_bf16_tile<256, 256, 2, 2, 64, 2>(p, dev, stream, 1, splits);
@@ -473,6 +478,7 @@ int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   g.group_m = 8;
   g.splits = 1;
   g.chunk_done = p.chunk_done;
+  g.slice_ready = p.slice_ready; g.gate_ticks = p.gate_ticks;
   g_last_tiles_per_chunk = g.tiles_m * g.tiles_n;
   // Two of the four-wave workgroups fit a compute unit (as with the 128x128 bf16 kernel, see workgroups_per_unit), but
   // here a unit that holds two takes about 1.75 times as long over them as over one (measured: 512 tiles of 64x64 on
@@ -695,6 +701,35 @@ MS_API int ms_gemm_os_ws(const void *const *A_slices, const void *const *B_slice
   p.act = activation; p.res = residual; p.ldr = ldr; p.row_sum = row_sum; p.row_sumsq = row_sumsq;
   p.ws = workspace; p.ws_bytes = workspace ? workspace_bytes : 0;
   return run(p, stream);
+}
+
+__global__ void signal_set_kernel(unsigned *flag, unsigned value) {
+  // everything enqueued on the stream before this kernel has ended; the release makes it visible to whoever then reads the flag
+  __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+MS_API int ms_gemm_os_gated(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
+                            int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype,
+                            void *workspace, size_t workspace_bytes, unsigned *slice_ready, unsigned timeout_ms, void *stream) {
+  if (!slice_ready || (reinterpret_cast<uintptr_t>(slice_ready) & 3))
+    return fail(MS_ERR_ARG, "ms_gemm_os_gated: slice_ready must be a 4-byte aligned device pointer to S + 1 words");
+  if (timeout_ms == 0 || timeout_ms > 60000) return fail(MS_ERR_ARG, "ms_gemm_os_gated: timeout_ms %u outside [1, 60000]", timeout_ms);
+  void *c1[1] = {C};
+  Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
+  p.ws = workspace; p.ws_bytes = workspace ? workspace_bytes : 0;
+  p.slice_ready = slice_ready;
+  int device = 0, wall_khz = 0;
+  MS_HIP(hipGetDevice(&device));
+  MS_HIP(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, device));
+  p.gate_ticks = (unsigned long long)timeout_ms * (unsigned long long)(wall_khz > 0 ? wall_khz : 100000);      // ticks of wall_clock64()
+  return run(p, stream);
+}
+
+MS_API int ms_signal_set(unsigned *flag, unsigned value, void *stream) {
+  if (!flag || (reinterpret_cast<uintptr_t>(flag) & 3)) return fail(MS_ERR_ARG, "ms_signal_set: flag must be a 4-byte aligned device pointer");
+  hipLaunchKernelGGL(signal_set_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, flag, value);
+  MS_HIP(hipGetLastError());
+  return MS_OK;
 }
 
 MS_API int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,

@@ -214,6 +214,48 @@ def _chunk_dtype(out, out_dtype):
     return dt
 
 
+def gemm_os_gated(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Tensor], slice_ready: torch.Tensor,
+                  out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
+                  timeout_ms: int = 2000) -> torch.Tensor:
+    """gemm_os as ONE launch that may be enqueued before its slices have arrived (``ms_gemm_os_gated``): the kernel
+    reads slice s of A and of B only after ``slice_ready[s]`` has become non-zero, the way the reference's
+    output-stationary body multiplies slice k while slice k + 1 is still being gathered (MeshFlow_OS,
+    TensorParallel.py:163-171).  ``slice_ready`` is an int32 GPU tensor of S + 1 words: the flags (set them with
+    ``signal_set`` on the stream that fills the slice, after the fill) and, last, a status word that must be zero before
+    the call and reads 1 afterwards if a wait lasted longer than ``timeout_ms`` (the result is then void: check it with
+    ``gate_timed_out`` once the stream has been synchronised).  A producer that needs compute units of this device
+    only runs beside the waiting product when units have been reserved (``ms_set_reserved_cus``)."""
+    call = _prepare_os(A_slices, B_slices, out, out_dtype)
+    S = len(A_slices)
+    if not (isinstance(slice_ready, torch.Tensor) and slice_ready.is_cuda and slice_ready.dtype == torch.int32
+            and slice_ready.dim() == 1 and slice_ready.numel() == S + 1 and slice_ready.is_contiguous()
+            and slice_ready.device == call.device):
+        raise ValueError("slice_ready must be a contiguous int32 GPU tensor of S + 1 words on the operands' device")
+    ws_ptr, ws_bytes, _ws_keep = _ws_args(call.device)
+    with torch.cuda.device(call.device):
+        rc = _lib.load().ms_gemm_os_gated(*call.args, ws_ptr, ws_bytes, ctypes.c_void_p(slice_ready.data_ptr()),
+                                          int(timeout_ms), _stream())
+    _lib.check(rc)
+    return call.out
+
+
+def signal_set(flags: torch.Tensor, index: int, value: int = 1) -> None:
+    """``flags[index] = value`` on the current stream, after everything enqueued on it before, as a release at system
+    scope (``ms_signal_set``): the producer's half of ``gemm_os_gated``."""
+    if not (isinstance(flags, torch.Tensor) and flags.is_cuda and flags.dtype == torch.int32 and flags.dim() == 1 and flags.is_contiguous()):
+        raise ValueError("flags must be a contiguous int32 GPU vector")
+    if not 0 <= index < flags.numel():
+        raise IndexError(f"flag index {index} outside [0, {flags.numel()})")
+    with torch.cuda.device(flags.device):
+        rc = _lib.load().ms_signal_set(ctypes.c_void_p(flags.data_ptr() + 4 * index), int(value), _stream())
+    _lib.check(rc)
+
+
+def gate_timed_out(slice_ready: torch.Tensor) -> bool:
+    """Whether a ``gemm_os_gated`` call with these flags gave up waiting for a slice (synchronises with the device)."""
+    return bool(slice_ready[-1].item() != 0)
+
+
 def gemm_ls(A: torch.Tensor, W_slices: Sequence[torch.Tensor],
             out: Optional[List[torch.Tensor]] = None, out_dtype: Optional[torch.dtype] = None) -> List[torch.Tensor]:
     """``Y_s = A @ W_s^T``, W_s stored ``[n_slice, k]``.  Chunks are fp32 by default (exact partial sums for
