@@ -392,10 +392,13 @@ def main():
             pack_slices(Wown, S, 8, 0, out=ws)
             ms.gemm_os(A, B, out=C)
         torch.matmul(X, W)
-        t_plain, t_gelu, t_sep, t_vendor, t_step = _legs([
+        # the same product behind its input gate with every slice already flagged: what the gate itself costs
+        flags = torch.ones(S + 1, dtype=torch.int32, device=C.device); flags[S] = 0
+        t_plain, t_gelu, t_sep, t_vendor, t_step, t_gated = _legs([
             lambda: ms.gemm_os(A, B, out=C), lambda: ms.gemm_os(A, B, out=C, activation="gelu"),
             lambda: torch.nn.functional.gelu(ms.gemm_os(A, B, out=C), approximate="tanh"),
-            lambda: torch.matmul(X, W), _device_step])
+            lambda: torch.matmul(X, W), _device_step, lambda: ms.gemm_os_gated(A, B, flags, out=C)])
+        extra["os_s4_gated_all_slices_flagged_ms"] = round(t_gated, 4)
         extra["os_s4_fused_gelu_ms"] = round(t_gelu, 4)
         extra["os_s4_then_separate_gelu_ms"] = round(t_sep, 4)
         extra["vendor_library_matmul_s1_ms"] = round(t_vendor, 4)

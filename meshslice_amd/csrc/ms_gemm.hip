@@ -419,7 +419,8 @@ int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
   if (g_variant != 0) return launch_variant(g_variant, g_splits > 1 ? g_splits : 1, p, dev, stream);
   const Pick single = pick_variant(p, dev);
-  if (p.flow == OS && single.splits == 1 && g_splits == 0) {
+  // (a gated product stays one launch: a second one would stand in the stream behind the first while that waits for slices)
+  if (p.flow == OS && single.splits == 1 && g_splits == 0 && !p.slice_ready) {
     constexpr int BM = 256, BN = 384;
     constexpr double EFF = 1.15;
     const long tiles_m = (p.M + BM - 1) / BM;
