@@ -127,6 +127,49 @@ def MeshFlow_OS(X, W, i, j, R, C, K, B):
     return local_gemm.gemm_os(A_slices, B_slices)
 
 
+_gather_streams = {}
+OVERLAP_RESERVED_CUS = 32      # compute units left to the emulated gathers' copy kernels beside the waiting product
+
+
+def MeshFlow_OS_overlap(X, W, i, j, R, C, K, B):
+    """MeshFlow_OS in the order the reference's schedule runs it (:163-171): the product is launched once, before any
+    slice has arrived, and multiplies slice k while the gathers of the later slices are still under way
+    (``gemm_os_gated``).  The emulated gather stream fills slice k of both operands, peer by peer, and raises flag k;
+    on a real mesh that stream is the collective's.  Same result as MeshFlow_OS, bit for bit."""
+    if K == 1:
+        raise ValueError("the sliced OS body is undefined for K == 1 (the reference adds slice 0 twice); "
+                         "use algorithm='collective' for the unsliced product")
+    px = [X[i][jj] for jj in range(C)]; pw = [W[ii][j] for ii in range(R)]
+    r, c = px[0].shape; h, n = pw[0].shape
+    _need(c, K * B, "sliced extent"); _need(h, K * B, "sliced extent")
+    w, hk = c // K, h // K
+    dev = px[0].device
+    bufA = torch.empty((K, r, C * w), dtype=px[0].dtype, device=dev)
+    bufB = torch.empty((K, R * hk, n), dtype=pw[0].dtype, device=dev)
+    ready = torch.zeros(K + 1, dtype=torch.int32, device=dev)
+    lib = local_gemm._lib.load()
+    cur = torch.cuda.current_stream(dev)
+    gather = _gather_streams.setdefault(dev, torch.cuda.Stream(dev))
+    gather.wait_stream(cur)                              # the flags are cleared and the shards are there
+    try:
+        lib.ms_set_reserved_cus(OVERLAP_RESERVED_CUS)
+        out = local_gemm.gemm_os_gated([bufA[k] for k in range(K)], [bufB[k] for k in range(K)], ready)
+    finally:
+        lib.ms_set_reserved_cus(0)
+    with torch.cuda.stream(gather):
+        for k in range(K):
+            # slice k of a shard: its B-wide blocks b with b % K == k (reference :155-158)
+            for p, blk in enumerate(px):
+                bufA[k][:, p * w:(p + 1) * w].copy_(blk.reshape(r, w // B, K, B)[:, :, k, :].reshape(r, w))
+            for p, blk in enumerate(pw):
+                bufB[k][p * hk:(p + 1) * hk].copy_(blk.reshape(hk // B, K, B, n)[:, k].reshape(hk, n))
+            local_gemm.signal_set(ready, k)
+    cur.wait_stream(gather)
+    if local_gemm.gate_timed_out(ready):
+        raise local_gemm._lib.MeshSliceError("the gated product gave up waiting for a slice: the gathers did not run beside it")
+    return out
+
+
 def MeshFlow_LS(X, W, i, j, R, C, K, B):
     """reference :174-193: K gathered row slices of W; K fp32 partial chunks X_ij @ W_k^T."""
     W_slices = _gather_row_slices([W[ii][j] for ii in range(R)], K, B)
@@ -361,6 +404,9 @@ class SPMD:
             assert mesh.devices.shape[0] == mesh.devices.shape[1], "cannon needs a square mesh"
             self.funcs = {"os": Cannon_OS, "ls": Cannon_LS, "rs": Cannon_RS}
             self.sliced = False
+        elif algorithm == "meshflow_overlap":      # MeshFlow with the OS product launched ahead of its gathers
+            self.funcs = {"os": MeshFlow_OS_overlap, "ls": MeshFlow_LS, "rs": MeshFlow_RS}
+            self.sliced = True
         else:  # like the reference, any other name selects the sliced MeshFlow bodies
             self.funcs = {"os": MeshFlow_OS, "ls": MeshFlow_LS, "rs": MeshFlow_RS}
             self.sliced = True

@@ -124,3 +124,25 @@ def test_the_gated_call_checks_its_arguments():
     ms.signal_set(good, S, 5)
     torch.cuda.synchronize()
     assert good.tolist() == [1, 1, 5]
+
+
+def test_the_mesh_body_that_launches_the_product_ahead_of_its_gathers_equals_meshflow():
+    """SPMD(mesh, 'meshflow_overlap').OS(K): every device launches its gated product first and fills the gathered slices
+    afterwards on a second stream, slice by slice; the global result equals MeshFlow's bit for bit."""
+    from meshslice_amd import TensorParallel as TP
+    from meshslice_amd.mesh import Mesh, create_device_mesh
+    mesh = Mesh(create_device_mesh((2, 2)), ("x", "y"))
+    X = _rand((512, 1024), 21, torch.bfloat16); W = _rand((1024, 768), 22, torch.bfloat16, 0.05)
+    lib = _lib.load()
+    try:
+        # (the overlapped body leaves compute units to its gathers; the tile choice, and with it the order of the
+        # additions, follows the units a product may use)
+        assert lib.ms_set_reserved_cus(TP.OVERLAP_RESERVED_CUS) == 0
+        want = TP.SPMD(mesh, "meshflow").OS(4)(X, W)
+    finally:
+        lib.ms_set_reserved_cus(0)
+    got = TP.SPMD(mesh, "meshflow_overlap").OS(4)(X, W)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    plain = TP.SPMD(mesh, "meshflow").OS(4)(X, W)
+    assert orc.rel_frobenius(got.float().cpu().numpy(), plain.float().cpu().numpy()) <= 1e-2
