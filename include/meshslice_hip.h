@@ -321,7 +321,7 @@ int ms_probe_l2_lds_stream(const void *buffer, size_t buffer_bytes, int region_s
                            int warmup, int reps, float *sink, float *ms_out, double *bytes_per_launch, void *stream);
 
 /* Hook for tests and measurements (thread-local): later bf16 calls on this thread use tile variant `variant % 100`
- * (1..13, 0 = the library's choice) and split the contraction `variant / 100` ways (2..8, 0 = the library's choice;
+ * (1..14, 0 = the library's choice) and split the contraction `variant / 100` ways (2..8, 0 = the library's choice;
  * a forced split needs a workspace and an output-stationary product).  Unknown ids are rejected with MS_ERR_ARG. */
 int ms_set_variant(int variant);
 

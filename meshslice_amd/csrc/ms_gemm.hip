@@ -34,6 +34,7 @@ MS_INSTANTIATE_RING(192, 256, 32, 4, 2, 2)
 MS_INSTANTIATE_RING(256, 256, 64, 2, 2, 4)
 MS_INSTANTIATE_RING(256, 192, 64, 2, 2, 2)
 MS_INSTANTIATE_RING(192, 256, 64, 2, 2, 2)
+MS_INSTANTIATE_RING(128, 128, 64, 3, 2, 2)
 #undef MS_INSTANTIATE_RING
 #define MS_INSTANTIATE_BIG(TM, TN)                                                                             \
   template __global__ void msk::gemm_bf16_big_kernel<TM, TN, true, false, true, false>(const msk::GemmArgs);   \
@@ -294,6 +295,8 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 //   7: 256x256, 8 waves, 2 x 64     8: 256x192, 4 waves, 2 x 64     9: 192x256, 4 waves, 2 x 64
 //  10: 256x384, 4 waves, 2 x 64 (gemm_bf16_big_kernel<4, 6>)     11: 384x192, 4 waves, 2 x 64 (gemm_bf16_big_kernel<6, 3>)
 //  12: 256x384, 4 waves, 2 x 64 on the 16x16x32 MFMA (gemm_bf16_x16_kernel)     13: 256x256, the same kernel
+//  14: 128x128, 4 waves, 3 x 64 (one workgroup per unit: for products of at most one round of such tiles, where a third
+//      stage covers the load latency that two 64-deep stages do not: 2048^3 in 20.7 us against 26.3 us, 1536^3 14.7 against 18.8)
 // The default picks the tile shape that wastes the least of the machine: a launch runs in
 // ceil(work items / CUs) rounds of one item per CU (a partly filled last round is charged in part, see
 // balanced_grid), so the estimate is rounds x tile area / relative tile
@@ -310,11 +313,11 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 // 2048 x 1536 x 12288 (64 tiles of 256x192): 170 us unsplit, 100 / 85 / 88 us with 2 / 3 / 4 splits.
 struct Pick { int v, splits; double cost; };
 
-constexpr int VARIANTS = 13;
+constexpr int VARIANTS = 14;
 struct TileShape { int bm, bn; };
 constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256}, {128, 128}, {256, 256}, {256, 192},
                                              {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192},
-                                             {256, 384}, {256, 256}};
+                                             {256, 384}, {256, 256}, {128, 128}};
 constexpr double X16_OVER_RING_256 = 1.10;   // unsplit 256x256: the 16x16x32 kernel (variant 13) against the eight-wave ring kernel (variant 7)
 constexpr int SPLIT_CHOICES[] = {1, 2, 3, 4, 6, 8};
 constexpr int SPLIT_MAX = 8;
@@ -353,7 +356,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   // prologue and write-out weigh most, and the one of the two that can split its contraction: 2048 x 2048 x 16384 in
   // 0.125 ms on 64 tiles x 4 splits, 0.165 ms on 256 tiles of 128x128; four waves stay selectable as variant 1)
   const bool rs = p.flow == RS, ls = p.flow == LS;
-  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.13 : ls ? 1.20 : 1.15}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, workgroups_per_unit(3) == 2 ? 0.42 : 0.55}};
+  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.13 : ls ? 1.20 : 1.15}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, workgroups_per_unit(3) == 2 ? 0.42 : 0.55}, {14, 0.66}};
   const long chunks = p.flow == OS ? 1 : p.S;
   const double total_k = p.flow == OS ? (double)p.K * p.S : (double)p.K;
   Pick best = {0, 1, 0};
@@ -405,6 +408,7 @@ int launch_variant(int v, int splits, const Problem &p, const DevFacts &dev, hip
     case 11: return launch_bf16_tile<384, 192, 2, 2, 64, 2, 1>(p, dev, stream, 11, splits);
     case 12: return launch_bf16_tile<256, 384, 2, 2, 64, 2, 2>(p, dev, stream, 12, splits);
     case 13: return launch_bf16_tile<256, 256, 2, 2, 64, 2, 2>(p, dev, stream, 13, splits);
+    case 14: return launch_bf16_tile<128, 128, 2, 2, 64, 3>(p, dev, stream, 14, splits);
     default: return fail(MS_ERR_ARG, "unknown kernel variant %d", v);
   }
 }

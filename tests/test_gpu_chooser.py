@@ -56,7 +56,7 @@ def test_default_choice_is_right_on_products_outside_the_gpt3_family(flow, shape
     assert lib.ms_set_variant(0) == 0
     run, check = operands(flow, shape)
     run()
-    assert 1 <= lib.ms_query(_lib.MS_QUERY_LAST_VARIANT) <= 13
+    assert 1 <= lib.ms_query(_lib.MS_QUERY_LAST_VARIANT) <= 14
     assert check() <= 1e-2
 
 

@@ -147,7 +147,7 @@ def _run_and_compare(flow, ops, dtype, tol, out_dtype=None):
     return err
 
 
-@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13])
+@pytest.mark.parametrize("variant", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14])
 @pytest.mark.parametrize("flow", ["os", "ls", "rs"])
 def test_bf16_random_cases_all_variants(flow, variant):
     _lib.check(_lib.load().ms_set_variant(variant))
@@ -161,7 +161,7 @@ def test_bf16_random_cases_all_variants(flow, variant):
         assert err < 1e-5
 
 
-@pytest.mark.parametrize("variant", [3, 7, 8, 10, 11, 12, 13])
+@pytest.mark.parametrize("variant", [3, 7, 8, 10, 11, 12, 13, 14])
 @pytest.mark.parametrize("flow", ["os", "rs"])
 def test_more_tiles_than_compute_units_with_a_partly_filled_last_round(flow, variant):
     """5120 x 5120 outputs are 280 to 1600 tiles, a whole number of rounds for none of the tile shapes on a device of
@@ -221,7 +221,7 @@ def test_bf16_output_is_one_rounding_of_the_fp32_accumulator():
     assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 3, 5, 8, 10, 11, 12, 13])
+@pytest.mark.parametrize("variant", [0, 1, 3, 5, 8, 10, 11, 12, 13, 14])
 @pytest.mark.parametrize("flow", ["ls", "rs"])
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
 def test_bf16_chunks_are_one_rounding_of_the_fp32_chunks(flow, variant, in_dtype):
@@ -484,7 +484,7 @@ def test_nan_and_inf_propagate():
 
 
 # ------------------------------------------------------------------ fused output-stationary epilogue
-@pytest.mark.parametrize("variant", [0, 1, 3, 4, 7, 8, 9, 10, 11, 12, 13])
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 7, 8, 9, 10, 11, 12, 13, 14])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_fused_epilogue_gelu_residual_moments(variant, out_dtype):
     """ms_gemm_os_fused: Y = gelu(sum_k A_k B_k) + residual, plus the row sums / sums of squares of Y
@@ -515,7 +515,7 @@ def test_fused_epilogue_gelu_residual_moments(variant, out_dtype):
     assert orc.rel_frobenius(host(s1b), host(plain).sum(1)) <= 1e-4
 
 
-@pytest.mark.parametrize("variant", [0, 3, 7, 8, 10, 11, 12, 13])
+@pytest.mark.parametrize("variant", [0, 3, 7, 8, 10, 11, 12, 13, 14])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 def test_one_call_per_slice_accumulating_in_place_through_the_residual(variant, out_dtype):
     """The output-stationary product slice by slice, as a mesh would issue it when each slice's call waits for that

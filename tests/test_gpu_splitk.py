@@ -151,7 +151,7 @@ def test_workspace_rules_of_the_c_abi():
     L.ms_set_variant(401)
     assert L.ms_gemm_os_ws(*head, *epi, ctypes.c_void_p(ws.data_ptr()), ws.numel(), None) == _lib.MS_ERR_ARG
     assert "no split path" in _lib.last_error()
-    assert L.ms_set_variant(108) == _lib.MS_ERR_ARG and L.ms_set_variant(908) == _lib.MS_ERR_ARG and L.ms_set_variant(14) == _lib.MS_ERR_ARG
+    assert L.ms_set_variant(108) == _lib.MS_ERR_ARG and L.ms_set_variant(908) == _lib.MS_ERR_ARG and L.ms_set_variant(15) == _lib.MS_ERR_ARG
     L.ms_set_variant(0)
     assert L.ms_workspace_init(None, 4096, None) == _lib.MS_ERR_ARG
     assert L.ms_workspace_init(ctypes.c_void_p(ws.data_ptr()), 100, None) == _lib.MS_ERR_ARG

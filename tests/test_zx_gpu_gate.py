@@ -30,7 +30,7 @@ def _slices(m, n, k, S, dtype, seed):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("variant", [0, 3, 7, 8, 9, 10, 11, 12, 13, 208])
+@pytest.mark.parametrize("variant", [0, 3, 7, 8, 9, 10, 11, 12, 13, 14, 208])
 def test_with_every_flag_set_the_gated_call_equals_the_plain_one(variant, dtype):
     if dtype == torch.float32 and variant:
         pytest.skip("tile variants are those of the bf16 kernels")

@@ -20,7 +20,7 @@ import test_gpu_signal as signal_tests
 
 pytestmark = [pytest.mark.gpu, pytest.mark.perf]
 SLACK = 1.15
-LAST_VARIANT = 13
+LAST_VARIANT = 14
 
 
 def _sustained(f, warm=10, steps=25):
