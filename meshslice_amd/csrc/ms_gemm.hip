@@ -301,7 +301,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 // ceil(work items / CUs) rounds of one item per CU (a partly filled last round is charged in part, see
 // balanced_grid), so the estimate is rounds x tile area / relative tile
 // efficiency (measured on the GPT-3-sized products, per flop, 256x256 = 1: the 256x384 tile, on the 16x16x32 kernel
-// that every such pick runs on, reaches 1.15 (OS) / 1.20 (LS) with a k-contiguous A and 1.13 without, the 384x192 tile 1.04 and 0.96,
+// that every such pick runs on, reaches 1.15 (OS) / 1.20 (LS) with a k-contiguous A and 1.16 without, the 384x192 tile 1.04,
 // 192-wide ring tiles about 0.93, 128x128 tiles about 0.55, or 0.42 per workgroup with two of them on a unit).  The ring-kernel defaults use four waves over two 64-deep stages when an operand is
 // k-contiguous: whole 128-byte lines per request, half as many barriers as 32-deep stages.
 //
@@ -318,7 +318,9 @@ struct TileShape { int bm, bn; };
 constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256}, {128, 128}, {256, 256}, {256, 192},
                                              {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192},
                                              {256, 384}, {256, 256}, {128, 128}};
-constexpr double X16_OVER_RING_256 = 1.10;   // unsplit 256x256: the 16x16x32 kernel (variant 13) against the eight-wave ring kernel (variant 7)
+// unsplit 256x256: the 16x16x32 kernel (variant 13) against the eight-wave ring kernel (variant 7); with two m/n-contiguous
+// operands (RS) it gains 0-6 % only
+constexpr double X16_OVER_RING_256 = 1.10, X16_OVER_RING_256_RS = 1.03;
 constexpr int SPLIT_CHOICES[] = {1, 2, 3, 4, 6, 8};
 constexpr int SPLIT_MAX = 8;
 constexpr long SPLIT_MIN_K = 512;            // contraction elements per split item, at least
@@ -356,7 +358,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   // prologue and write-out weigh most, and the one of the two that can split its contraction: 2048 x 2048 x 16384 in
   // 0.125 ms on 64 tiles x 4 splits, 0.165 ms on 256 tiles of 128x128; four waves stay selectable as variant 1)
   const bool rs = p.flow == RS, ls = p.flow == LS;
-  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.13 : ls ? 1.20 : 1.15}, {11, rs ? 0.96 : 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, workgroups_per_unit(3) == 2 ? 0.42 : 0.55}, {14, 0.66}};
+  const Cand cands[] = {{7, 1.0}, {10, rs ? 1.16 : ls ? 1.20 : 1.15}, {11, 1.04}, {rs ? 5 : 8, rs ? 0.95 : 0.93}, {rs ? 6 : 9, rs ? 0.95 : 0.93}, {3, workgroups_per_unit(3) == 2 ? 0.42 : 0.55}, {14, 0.66}};
   const long chunks = p.flow == OS ? 1 : p.S;
   const double total_k = p.flow == OS ? (double)p.K * p.S : (double)p.K;
   Pick best = {0, 1, 0};
@@ -377,7 +379,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
       const double exchange = splits == 1 ? 0.0 : (SPLIT_FIX + (double)splits * p.M * p.N * SPLIT_PER_ELEMENT) / total_k;
       // (a split 256x384 product stays on the 32x32x16 kernel, which carries the exchange and is about 5 % slower; an
       // unsplit 256x256 one runs on the 16x16x32 kernel, 7-14 % faster than the eight-wave ring kernel that carries the split)
-      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * X16_OVER_RING_256 : c.eff;
+      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * (rs ? X16_OVER_RING_256_RS : X16_OVER_RING_256) : c.eff;
       const double cost = rounds * bm * bn / eff / splits + exchange;
       if (best.v == 0 || cost < best.cost) best = {c.v, splits, cost};
     }
