@@ -319,8 +319,10 @@ constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256},
                                              {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192},
                                              {256, 384}, {256, 256}, {128, 128}};
 // unsplit 256x256: the 16x16x32 kernel (variant 13) against the eight-wave ring kernel (variant 7); with two m/n-contiguous
-// operands (RS) it gains 0-6 % only
+// operands (RS) it gains 0-6 % only, and beyond some 6000 contraction elements per chunk it loses (10240 x 2560 x 12288 in
+// two chunks: 0.622 against 0.555 ms), so there the ring kernel stays
 constexpr double X16_OVER_RING_256 = 1.10, X16_OVER_RING_256_RS = 1.03;
+constexpr int X16_RS_MAX_K = 6144;
 constexpr int SPLIT_CHOICES[] = {1, 2, 3, 4, 6, 8};
 constexpr int SPLIT_MAX = 8;
 constexpr long SPLIT_MIN_K = 512;            // contraction elements per split item, at least
@@ -379,7 +381,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
       const double exchange = splits == 1 ? 0.0 : (SPLIT_FIX + (double)splits * p.M * p.N * SPLIT_PER_ELEMENT) / total_k;
       // (a split 256x384 product stays on the 32x32x16 kernel, which carries the exchange and is about 5 % slower; an
       // unsplit 256x256 one runs on the 16x16x32 kernel, 7-14 % faster than the eight-wave ring kernel that carries the split)
-      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * (rs ? X16_OVER_RING_256_RS : X16_OVER_RING_256) : c.eff;
+      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * (!rs ? X16_OVER_RING_256 : p.K <= X16_RS_MAX_K ? X16_OVER_RING_256_RS : 1.0) : c.eff;
       const double cost = rounds * bm * bn / eff / splits + exchange;
       if (best.v == 0 || cost < best.cost) best = {c.v, splits, cost};
     }
@@ -389,7 +391,7 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   if (best.splits == 1 && best.v == 10) best.v = 12;
   // Likewise an unsplit 256x256 product (4096^3 in 0.093-0.095 ms against 0.106 ms on the ring kernel, 4096 x 4096 x 14336 in
   // 0.302-0.309 against 0.344 ms); the eight-wave ring kernel stays selectable as variant 7 and carries the split contraction.
-  if (best.splits == 1 && best.v == 7) best.v = 13;
+  if (best.splits == 1 && best.v == 7 && !(rs && p.K > X16_RS_MAX_K)) best.v = 13;
   return best;
 }
 
