@@ -321,7 +321,7 @@ constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256},
 // unsplit 256x256: the 16x16x32 kernel (variant 13) against the eight-wave ring kernel (variant 7); with two m/n-contiguous
 // operands (RS) it gains 0-6 % only, and beyond some 6000 contraction elements per chunk it loses (10240 x 2560 x 12288 in
 // two chunks: 0.622 against 0.555 ms), so there the ring kernel stays
-constexpr double X16_OVER_RING_256 = 1.10, X16_OVER_RING_256_RS = 1.03;
+constexpr double X16_OVER_RING_256 = 1.10, X16_OVER_RING_256_LS = 1.13, X16_OVER_RING_256_RS = 1.03;
 constexpr int X16_RS_MAX_K = 6144;
 constexpr int SPLIT_CHOICES[] = {1, 2, 3, 4, 6, 8};
 constexpr int SPLIT_MAX = 8;
@@ -377,11 +377,15 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
       const double whole = (double)((tiles * splits + slots - 1) / slots);
       // (the 128x128 kernel does not reach the power limit: its units gain no clock from idle neighbours)
       const double loss = c.v == 3 ? 1.0 : PARTIAL_ROUND_LOSS;
-      const double rounds = exact <= 1.0 ? 1.0 : exact + loss * (whole - exact);
+      // (a launch of less than one round on the hand-scheduled kernels, which sit on the power limit: the idle units'
+      // power lets the busy ones clock up to 1.4 times higher; the ring kernels' short launches are bound by latencies)
+      const bool power_bound = splits == 1 && (c.v == 7 || c.v == 10 || c.v == 11);
+      const double part = exact + loss * (1.0 - exact);
+      const double rounds = exact <= 1.0 ? (power_bound ? (part > 0.7 ? part : 0.7) : 1.0) : exact + loss * (whole - exact);
       const double exchange = splits == 1 ? 0.0 : (SPLIT_FIX + (double)splits * p.M * p.N * SPLIT_PER_ELEMENT) / total_k;
       // (a split 256x384 product stays on the 32x32x16 kernel, which carries the exchange and is about 5 % slower; an
       // unsplit 256x256 one runs on the 16x16x32 kernel, 7-14 % faster than the eight-wave ring kernel that carries the split)
-      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * (!rs ? X16_OVER_RING_256 : p.K <= X16_RS_MAX_K ? X16_OVER_RING_256_RS : 1.0) : c.eff;
+      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * (ls ? X16_OVER_RING_256_LS : !rs ? X16_OVER_RING_256 : p.K <= X16_RS_MAX_K ? X16_OVER_RING_256_RS : 1.0) : c.eff;
       const double cost = rounds * bm * bn / eff / splits + exchange;
       if (best.v == 0 || cost < best.cost) best = {c.v, splits, cost};
     }
