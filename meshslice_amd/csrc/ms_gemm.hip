@@ -375,17 +375,20 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
       const long slots = (long)dev.cus * (splits == 1 ? workgroups_per_unit(c.v) : 1);     // (a split launch is one item per unit)
       const double exact = (double)(tiles * splits) / slots;
       const double whole = (double)((tiles * splits + slots - 1) / slots);
-      // (the 128x128 kernel does not reach the power limit: its units gain no clock from idle neighbours)
-      const double loss = c.v == 3 ? 1.0 : PARTIAL_ROUND_LOSS;
-      // (a launch of less than one round on the hand-scheduled kernels, which sit on the power limit: the idle units'
-      // power lets the busy ones clock up to 1.4 times higher; the ring kernels' short launches are bound by latencies)
-      const bool power_bound = splits == 1 && (c.v == 7 || c.v == 10 || c.v == 11);
+      // (the 128x128 kernels do not reach the power limit: their units gain no clock from idle neighbours)
+      const bool small_tile = c.v == 3 || c.v == 14;
+      const double loss = small_tile ? 1.0 : PARTIAL_ROUND_LOSS;
+      // (a launch of less than one round is charged the same way, down to 0.7 of a round: the idle units' power lets the
+      // busy ones clock up to 1.4 times higher)
       const double part = exact + loss * (1.0 - exact);
-      const double rounds = exact <= 1.0 ? (power_bound ? (part > 0.7 ? part : 0.7) : 1.0) : exact + loss * (whole - exact);
+      const double rounds = exact <= 1.0 ? (part > 0.7 ? part : 0.7) : exact + loss * (whole - exact);
       const double exchange = splits == 1 ? 0.0 : (SPLIT_FIX + (double)splits * p.M * p.N * SPLIT_PER_ELEMENT) / total_k;
       // (a split 256x384 product stays on the 32x32x16 kernel, which carries the exchange and is about 5 % slower; an
       // unsplit 256x256 one runs on the 16x16x32 kernel, 7-14 % faster than the eight-wave ring kernel that carries the split)
-      const double eff = c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * (ls ? X16_OVER_RING_256_LS : !rs ? X16_OVER_RING_256 : p.K <= X16_RS_MAX_K ? X16_OVER_RING_256_RS : 1.0) : c.eff;
+      // (two 128x128 workgroups share a unit only where there are more tiles than units: 0.55 alone, 0.42 each when every
+      // unit holds two)
+      const double shared = c.v == 3 && workgroups_per_unit(3) == 2 ? (tiles * splits <= dev.cus ? 0.0 : tiles * splits >= 2L * dev.cus ? 1.0 : (double)(tiles * splits - dev.cus) / dev.cus) : 0.0;
+      const double eff = c.v == 3 && workgroups_per_unit(3) == 2 ? 0.55 - 0.13 * shared : c.v == 10 && splits > 1 ? c.eff / 1.05 : c.v == 7 && splits == 1 ? c.eff * (ls ? X16_OVER_RING_256_LS : !rs ? X16_OVER_RING_256 : p.K <= X16_RS_MAX_K ? X16_OVER_RING_256_RS : 1.0) : c.eff;
       const double cost = rounds * bm * bn / eff / splits + exchange;
       if (best.v == 0 || cost < best.cost) best = {c.v, splits, cost};
     }
@@ -395,7 +398,10 @@ Pick pick_variant(const Problem &p, const DevFacts &dev) {
   if (best.splits == 1 && best.v == 10) best.v = 12;
   // Likewise an unsplit 256x256 product (4096^3 in 0.093-0.095 ms against 0.106 ms on the ring kernel, 4096 x 4096 x 14336 in
   // 0.302-0.309 against 0.344 ms); the eight-wave ring kernel stays selectable as variant 7 and carries the split contraction.
-  if (best.splits == 1 && best.v == 7 && !(rs && p.K > X16_RS_MAX_K)) best.v = 13;
+  // (not where an LS chunk is a single tile column: every XCD then streams all of A, the product is bound by the fabric, and
+  // two waves per SIMD ride that out better: 8192 x 256 x 8192 in eight chunks 0.217 against 0.262 ms)
+  const bool one_column_chunks = ls && p.N <= 256;
+  if (best.splits == 1 && best.v == 7 && !(rs && p.K > X16_RS_MAX_K) && !one_column_chunks) best.v = 13;
   return best;
 }
 
