@@ -210,8 +210,26 @@ int ms_gemm_os_gated(const void *const *A_slices, const void *const *B_slices, i
                      void *workspace, size_t workspace_bytes,
                      unsigned *slice_ready, unsigned timeout_ms, void *stream);
 
+/* ms_gemm_ls_signal / ms_gemm_rs_signal behind the same gate: the kernel reads the gathered operand slice of chunk s
+ * (W_s, X_s) only after slice_ready[s] has become non-zero, as MeshFlow_LS / MeshFlow_RS gather slice k + 1 while chunk k
+ * is being multiplied (TensorParallel.py:176-189, :198-212); the stationary operand (A, W) is read from the start.
+ * slice_ready and timeout_ms as in ms_gemm_os_gated (S flags and the status word).  chunk_done and tiles_per_chunk may
+ * both be NULL (no completion counters); with them one launch has both ends open: slices arrive while it runs, and chunks
+ * are handed on as they complete.  The tile list is chunk-major, so a launch of more workgroups than one chunk has
+ * tiles starts on several chunks at once and each workgroup waits for its own chunk's slice. */
+int ms_gemm_ls_gated(const void *A, int lda, const void *const *W_slices, int ldw, int S,
+                     int m, int n_slice, int k,
+                     void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
+                     unsigned *chunk_done, int *tiles_per_chunk,
+                     unsigned *slice_ready, unsigned timeout_ms, void *stream);
+int ms_gemm_rs_gated(const void *const *X_slices, int ldx, const void *W, int ldw, int S,
+                     int m_slice, int n, int k,
+                     void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
+                     unsigned *chunk_done, int *tiles_per_chunk,
+                     unsigned *slice_ready, unsigned timeout_ms, void *stream);
+
 /* Sets *flag = value (device memory) once everything enqueued on `stream` before the call has completed, as a release
- * at system scope: the producer's half of ms_gemm_os_gated (and a way to clear or preset flags in stream order).  No
+ * at system scope: the producer's half of the gated calls (and a way to clear or preset flags in stream order).  No
  * counterpart in the reference, where XLA orders the gathers and the einsums. */
 int ms_signal_set(unsigned *flag, unsigned value, void *stream);
 

@@ -131,21 +131,37 @@ _gather_streams = {}
 OVERLAP_RESERVED_CUS = 32      # compute units left to the emulated gathers' copy kernels beside the waiting product
 
 
-def MeshFlow_OS_overlap(X, W, i, j, R, C, K, B):
-    """MeshFlow_OS in the order the reference's schedule runs it (:163-171): the product is launched once, before any
-    slice has arrived, and multiplies slice k while the gathers of the later slices are still under way
-    (``gemm_os_gated``).  The emulated gather stream fills slice k of both operands, peer by peer, and raises flag k;
-    on a real mesh that stream is the collective's.  Same result as MeshFlow_OS, bit for bit."""
-    if K == 1:
-        raise ValueError("the sliced OS body is undefined for K == 1 (the reference adds slice 0 twice); "
-                         "use algorithm='collective' for the unsliced product")
-    px = [X[i][jj] for jj in range(C)]; pw = [W[ii][j] for ii in range(R)]
-    r, c = px[0].shape; h, n = pw[0].shape
-    _need(c, K * B, "sliced extent"); _need(h, K * B, "sliced extent")
-    w, hk = c // K, h // K
-    dev = px[0].device
-    bufA = torch.empty((K, r, C * w), dtype=px[0].dtype, device=dev)
-    bufB = torch.empty((K, R * hk, n), dtype=pw[0].dtype, device=dev)
+def _col_slice_filler(peers, K, B):
+    """(buffer ``[K, rows, len(peers) * cols / K]`` for the K gathered column slices, ``fill(k)`` that gathers slice k into
+    it on the current stream): slice k of a shard is its B-wide column blocks b with b % K == k (reference :155,157,198-199)."""
+    r, c = peers[0].shape
+    _need(c, K * B, "sliced extent")
+    w = c // K
+    buf = torch.empty((K, r, len(peers) * w), dtype=peers[0].dtype, device=peers[0].device)
+
+    def fill(k):
+        for p, blk in enumerate(peers):
+            buf[k][:, p * w:(p + 1) * w].copy_(blk.reshape(r, w // B, K, B)[:, :, k, :].reshape(r, w))
+    return buf, fill
+
+
+def _row_slice_filler(peers, K, B):
+    """The same for the K gathered row slices ``[K, len(peers) * rows / K, cols]`` (reference :156,158,177-178)."""
+    h, n = peers[0].shape
+    _need(h, K * B, "sliced extent")
+    hk = h // K
+    buf = torch.empty((K, len(peers) * hk, n), dtype=peers[0].dtype, device=peers[0].device)
+
+    def fill(k):
+        for p, blk in enumerate(peers):
+            buf[k][p * hk:(p + 1) * hk].copy_(blk.reshape(hk // B, K, B, n)[:, k].reshape(hk, n))
+    return buf, fill
+
+
+def _launch_ahead_of_gathers(K, dev, launch, fills):
+    """``launch(ready)`` enqueues the gated product on the current stream with all K flags down; the emulated gather
+    stream then fills slice after slice (``fills``: one callable per gathered operand) and raises its flag.  On a real
+    mesh that stream is the collective's."""
     ready = torch.zeros(K + 1, dtype=torch.int32, device=dev)
     lib = local_gemm._lib.load()
     cur = torch.cuda.current_stream(dev)
@@ -153,21 +169,47 @@ def MeshFlow_OS_overlap(X, W, i, j, R, C, K, B):
     gather.wait_stream(cur)                              # the flags are cleared and the shards are there
     try:
         lib.ms_set_reserved_cus(OVERLAP_RESERVED_CUS)
-        out = local_gemm.gemm_os_gated([bufA[k] for k in range(K)], [bufB[k] for k in range(K)], ready)
+        out = launch(ready)
     finally:
         lib.ms_set_reserved_cus(0)
     with torch.cuda.stream(gather):
         for k in range(K):
-            # slice k of a shard: its B-wide blocks b with b % K == k (reference :155-158)
-            for p, blk in enumerate(px):
-                bufA[k][:, p * w:(p + 1) * w].copy_(blk.reshape(r, w // B, K, B)[:, :, k, :].reshape(r, w))
-            for p, blk in enumerate(pw):
-                bufB[k][p * hk:(p + 1) * hk].copy_(blk.reshape(hk // B, K, B, n)[:, k].reshape(hk, n))
+            for fill in fills:
+                fill(k)
             local_gemm.signal_set(ready, k)
     cur.wait_stream(gather)
     if local_gemm.gate_timed_out(ready):
         raise local_gemm._lib.MeshSliceError("the gated product gave up waiting for a slice: the gathers did not run beside it")
     return out
+
+
+def MeshFlow_OS_overlap(X, W, i, j, R, C, K, B):
+    """MeshFlow_OS in the order the reference's schedule runs it (:163-171): the product is launched once, before any
+    slice has arrived, and multiplies slice k while the gathers of the later slices are still under way
+    (``gemm_os_gated``).  The emulated gather stream fills slice k of both operands, peer by peer, and raises flag k.
+    Same result as MeshFlow_OS, bit for bit."""
+    if K == 1:
+        raise ValueError("the sliced OS body is undefined for K == 1 (the reference adds slice 0 twice); "
+                         "use algorithm='collective' for the unsliced product")
+    bufA, fillA = _col_slice_filler([X[i][jj] for jj in range(C)], K, B)
+    bufB, fillB = _row_slice_filler([W[ii][j] for ii in range(R)], K, B)
+    return _launch_ahead_of_gathers(K, bufA.device, lambda ready: local_gemm.gemm_os_gated([bufA[k] for k in range(K)], [bufB[k] for k in range(K)], ready),
+                                    (fillA, fillB))
+
+
+def MeshFlow_LS_overlap(X, W, i, j, R, C, K, B):
+    """MeshFlow_LS with the one launch ahead of the gathers of W's row slices (:176-189; ``gemm_ls_gated``): chunk k is
+    multiplied as soon as slice k has arrived.  Same chunks as MeshFlow_LS, bit for bit."""
+    bufW, fillW = _row_slice_filler([W[ii][j] for ii in range(R)], K, B)
+    own = _own(X[i][j])
+    return _launch_ahead_of_gathers(K, bufW.device, lambda ready: local_gemm.gemm_ls_gated(own, [bufW[k] for k in range(K)], ready), (fillW,))
+
+
+def MeshFlow_RS_overlap(X, W, i, j, R, C, K, B):
+    """MeshFlow_RS with the one launch ahead of the gathers of X's column slices (:198-212; ``gemm_rs_gated``)."""
+    bufX, fillX = _col_slice_filler([X[i][jj] for jj in range(C)], K, B)
+    own = _own(W[i][j])
+    return _launch_ahead_of_gathers(K, bufX.device, lambda ready: local_gemm.gemm_rs_gated([bufX[k] for k in range(K)], own, ready), (fillX,))
 
 
 def MeshFlow_LS(X, W, i, j, R, C, K, B):
@@ -404,8 +446,8 @@ class SPMD:
             assert mesh.devices.shape[0] == mesh.devices.shape[1], "cannon needs a square mesh"
             self.funcs = {"os": Cannon_OS, "ls": Cannon_LS, "rs": Cannon_RS}
             self.sliced = False
-        elif algorithm == "meshflow_overlap":      # MeshFlow with the OS product launched ahead of its gathers
-            self.funcs = {"os": MeshFlow_OS_overlap, "ls": MeshFlow_LS, "rs": MeshFlow_RS}
+        elif algorithm == "meshflow_overlap":      # MeshFlow with each device's one product launched ahead of its gathers
+            self.funcs = {"os": MeshFlow_OS_overlap, "ls": MeshFlow_LS_overlap, "rs": MeshFlow_RS_overlap}
             self.sliced = True
         else:  # like the reference, any other name selects the sliced MeshFlow bodies
             self.funcs = {"os": MeshFlow_OS, "ls": MeshFlow_LS, "rs": MeshFlow_RS}

@@ -35,7 +35,7 @@ LIB_PATH = os.path.join(_HERE, "libmeshslice_hip.so")
 
 EXPORTS = (
     "ms_version", "ms_last_error", "ms_query", "ms_set_variant",
-    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_os_ws", "ms_gemm_os_noalloc", "ms_gemm_os_gated", "ms_signal_set", "ms_workspace_bytes", "ms_workspace_init", "ms_time_os_ws", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_gemm_ls_signal", "ms_gemm_rs_signal", "ms_set_reserved_cus",
+    "ms_gemm_os", "ms_gemm_os_fused", "ms_gemm_os_ws", "ms_gemm_os_noalloc", "ms_gemm_os_gated", "ms_gemm_ls_gated", "ms_gemm_rs_gated", "ms_signal_set", "ms_workspace_bytes", "ms_workspace_init", "ms_time_os_ws", "ms_gemm_ls", "ms_gemm_rs", "ms_gemm_ls_ex", "ms_gemm_rs_ex", "ms_gemm_ls_signal", "ms_gemm_rs_signal", "ms_set_reserved_cus",
     "ms_time_os", "ms_time_ls", "ms_time_rs", "ms_time_ls_ex", "ms_time_rs_ex",
     "ms_pack_slices", "ms_unpack_chunks", "ms_probe_mfma_stream", "ms_probe_mfma_stream_ex",
     "ms_probe_os_parts", "ms_probe_l2_lds_stream",
@@ -77,6 +77,11 @@ def _declare(lib):
     # ..., out_dtype, workspace, workspace_bytes, slice_ready, timeout_ms, stream
     lib.ms_gemm_os_gated.argtypes = os_args[:-1] + [c_vp, ctypes.c_size_t, c_vp, ctypes.c_uint, c_vp]
     lib.ms_gemm_os_gated.restype = c_int
+    # ..., in_dtype, out_dtype, chunk_done, tiles_per_chunk, slice_ready, timeout_ms, stream
+    lib.ms_gemm_ls_gated.argtypes = ls_args[:-1] + [c_int, c_vp, ctypes.POINTER(c_int), c_vp, ctypes.c_uint, c_vp]
+    lib.ms_gemm_ls_gated.restype = c_int
+    lib.ms_gemm_rs_gated.argtypes = rs_args[:-1] + [c_int, c_vp, ctypes.POINTER(c_int), c_vp, ctypes.c_uint, c_vp]
+    lib.ms_gemm_rs_gated.restype = c_int
     lib.ms_signal_set.argtypes = [c_vp, ctypes.c_uint, c_vp]
     lib.ms_signal_set.restype = c_int
     lib.ms_time_os_ws.argtypes = os_args[:-1] + [c_vp, ctypes.c_size_t, c_vp, c_int, c_int, fp]

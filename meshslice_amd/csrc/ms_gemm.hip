@@ -727,21 +727,29 @@ __global__ void signal_set_kernel(unsigned *flag, unsigned value) {
   __hip_atomic_store(flag, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
-MS_API int ms_gemm_os_gated(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
-                            int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype,
-                            void *workspace, size_t workspace_bytes, unsigned *slice_ready, unsigned timeout_ms, void *stream) {
+// the gate's half of a Problem: the flags, and the longest wait for one of them in ticks of wall_clock64()
+namespace {
+int set_gate(Problem &p, unsigned *slice_ready, unsigned timeout_ms, const char *fn) {
   if (!slice_ready || (reinterpret_cast<uintptr_t>(slice_ready) & 3))
-    return fail(MS_ERR_ARG, "ms_gemm_os_gated: slice_ready must be a 4-byte aligned device pointer to S + 1 words");
-  if (timeout_ms == 0 || timeout_ms > 60000) return fail(MS_ERR_ARG, "ms_gemm_os_gated: timeout_ms %u outside [1, 60000]", timeout_ms);
-  void *c1[1] = {C};
-  Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
-  p.ws = workspace; p.ws_bytes = workspace ? workspace_bytes : 0;
+    return fail(MS_ERR_ARG, "%s: slice_ready must be a 4-byte aligned device pointer to S + 1 words", fn);
+  if (timeout_ms == 0 || timeout_ms > 60000) return fail(MS_ERR_ARG, "%s: timeout_ms %u outside [1, 60000]", fn, timeout_ms);
   p.slice_ready = slice_ready;
   int device = 0, wall_khz = 0;
   MS_HIP(hipGetDevice(&device));
   MS_HIP(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, device));
-  p.gate_ticks = (unsigned long long)timeout_ms * (unsigned long long)(wall_khz > 0 ? wall_khz : 100000);      // ticks of wall_clock64()
-  return run(p, stream);
+  p.gate_ticks = (unsigned long long)timeout_ms * (unsigned long long)(wall_khz > 0 ? wall_khz : 100000);
+  return MS_OK;
+}
+}  // namespace
+
+MS_API int ms_gemm_os_gated(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,
+                            int lda, int ldb, void *C, int ldc, int in_dtype, int out_dtype,
+                            void *workspace, size_t workspace_bytes, unsigned *slice_ready, unsigned timeout_ms, void *stream) {
+  void *c1[1] = {C};
+  Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
+  p.ws = workspace; p.ws_bytes = workspace ? workspace_bytes : 0;
+  const int rc = set_gate(p, slice_ready, timeout_ms, "ms_gemm_os_gated");
+  return rc ? rc : run(p, stream);
 }
 
 MS_API int ms_signal_set(unsigned *flag, unsigned value, void *stream) {
@@ -852,6 +860,32 @@ MS_API int ms_gemm_rs_signal(const void *const *X_slices, int ldx, const void *W
                              unsigned *chunk_done, int *tiles_per_chunk, void *stream) {
   const void *w1[1] = {W};
   return run_signal(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype, out_dtype), chunk_done, tiles_per_chunk, stream, "ms_gemm_rs_signal");
+}
+
+// the chunk-producing calls behind the input gate; the completion counters are optional here
+namespace {
+int run_chunks_gated(Problem p, unsigned *chunk_done, int *tiles_per_chunk, unsigned *slice_ready, unsigned timeout_ms, void *stream, const char *fn) {
+  if ((chunk_done == nullptr) != (tiles_per_chunk == nullptr)) return fail(MS_ERR_ARG, "%s: chunk_done and tiles_per_chunk come together or not at all", fn);
+  const int rc = set_gate(p, slice_ready, timeout_ms, fn);
+  if (rc) return rc;
+  return chunk_done ? run_signal(p, chunk_done, tiles_per_chunk, stream, fn) : run(p, stream);
+}
+}  // namespace
+
+MS_API int ms_gemm_ls_gated(const void *A, int lda, const void *const *W_slices, int ldw, int S, int m, int n_slice, int k,
+                            void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
+                            unsigned *chunk_done, int *tiles_per_chunk, unsigned *slice_ready, unsigned timeout_ms, void *stream) {
+  const void *a1[1] = {A};
+  return run_chunks_gated(make_ls(a1, lda, W_slices, ldw, S, m, n_slice, k, Y_chunks, ldy, in_dtype, out_dtype), chunk_done, tiles_per_chunk,
+                          slice_ready, timeout_ms, stream, "ms_gemm_ls_gated");
+}
+
+MS_API int ms_gemm_rs_gated(const void *const *X_slices, int ldx, const void *W, int ldw, int S, int m_slice, int n, int k,
+                            void *const *Y_chunks, int ldy, int in_dtype, int out_dtype,
+                            unsigned *chunk_done, int *tiles_per_chunk, unsigned *slice_ready, unsigned timeout_ms, void *stream) {
+  const void *w1[1] = {W};
+  return run_chunks_gated(make_rs(X_slices, ldx, w1, ldw, S, m_slice, n, k, Y_chunks, ldy, in_dtype, out_dtype), chunk_done, tiles_per_chunk,
+                          slice_ready, timeout_ms, stream, "ms_gemm_rs_gated");
 }
 
 MS_API int ms_time_os(const void *const *A_slices, const void *const *B_slices, int S, int m, int n, int k_slice,

@@ -226,11 +226,7 @@ def gemm_os_gated(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Ten
     ``gate_timed_out`` once the stream has been synchronised).  A producer that needs compute units of this device
     only runs beside the waiting product when units have been reserved (``ms_set_reserved_cus``)."""
     call = _prepare_os(A_slices, B_slices, out, out_dtype)
-    S = len(A_slices)
-    if not (isinstance(slice_ready, torch.Tensor) and slice_ready.is_cuda and slice_ready.dtype == torch.int32
-            and slice_ready.dim() == 1 and slice_ready.numel() == S + 1 and slice_ready.is_contiguous()
-            and slice_ready.device == call.device):
-        raise ValueError("slice_ready must be a contiguous int32 GPU tensor of S + 1 words on the operands' device")
+    _check_flags(slice_ready, len(A_slices), call.device)
     ws_ptr, ws_bytes, _ws_keep = _ws_args(call.device)
     with torch.cuda.device(call.device):
         rc = _lib.load().ms_gemm_os_gated(*call.args, ws_ptr, ws_bytes, ctypes.c_void_p(slice_ready.data_ptr()),
@@ -239,9 +235,47 @@ def gemm_os_gated(A_slices: Sequence[torch.Tensor], B_slices: Sequence[torch.Ten
     return call.out
 
 
+def _check_flags(slice_ready, S, device):
+    if not (isinstance(slice_ready, torch.Tensor) and slice_ready.is_cuda and slice_ready.dtype == torch.int32
+            and slice_ready.dim() == 1 and slice_ready.numel() == S + 1 and slice_ready.is_contiguous()
+            and slice_ready.device == device):
+        raise ValueError("slice_ready must be a contiguous int32 GPU tensor of S + 1 words on the operands' device")
+
+
+def _chunks_gated(entry, call, S, slice_ready, chunk_done, timeout_ms):
+    _check_flags(slice_ready, S, call.device)
+    tiles = ctypes.c_int(0)
+    if chunk_done is not None:
+        _check_counters(chunk_done, S, call.device)
+    with torch.cuda.device(call.device):
+        rc = entry(*call.args, ctypes.c_void_p(chunk_done.data_ptr()) if chunk_done is not None else None,
+                   ctypes.byref(tiles) if chunk_done is not None else None,
+                   ctypes.c_void_p(slice_ready.data_ptr()), int(timeout_ms), _stream())
+    _lib.check(rc)
+    return call.out if chunk_done is None else (call.out, tiles.value)
+
+
+def gemm_ls_gated(A: torch.Tensor, W_slices: Sequence[torch.Tensor], slice_ready: torch.Tensor,
+                  out: Optional[List[torch.Tensor]] = None, out_dtype: Optional[torch.dtype] = None,
+                  chunk_done: Optional[torch.Tensor] = None, timeout_ms: int = 2000):
+    """gemm_ls as one launch that may be enqueued before the weight slices have arrived (``ms_gemm_ls_gated``): ``W_s`` is
+    read only after ``slice_ready[s]`` has become non-zero (MeshFlow_LS gathers slice k + 1 while chunk k is multiplied,
+    TensorParallel.py:176-189); flags, status word and time limit as for ``gemm_os_gated``.  With ``chunk_done`` (see
+    ``gemm_ls_signal``) the call also counts finished tiles per chunk and returns ``(chunks, tiles_per_chunk)``."""
+    return _chunks_gated(_lib.load().ms_gemm_ls_gated, _prepare_ls(A, W_slices, out, out_dtype), len(W_slices), slice_ready, chunk_done, timeout_ms)
+
+
+def gemm_rs_gated(X_slices: Sequence[torch.Tensor], W: torch.Tensor, slice_ready: torch.Tensor,
+                  out: Optional[List[torch.Tensor]] = None, out_dtype: Optional[torch.dtype] = None,
+                  chunk_done: Optional[torch.Tensor] = None, timeout_ms: int = 2000):
+    """gemm_rs behind the input gate (``ms_gemm_rs_gated``; see gemm_ls_gated; reference TensorParallel.py:198-212):
+    ``X_s`` is read only after ``slice_ready[s]`` has become non-zero."""
+    return _chunks_gated(_lib.load().ms_gemm_rs_gated, _prepare_rs(X_slices, W, out, out_dtype), len(X_slices), slice_ready, chunk_done, timeout_ms)
+
+
 def signal_set(flags: torch.Tensor, index: int, value: int = 1) -> None:
     """``flags[index] = value`` on the current stream, after everything enqueued on it before, as a release at system
-    scope (``ms_signal_set``): the producer's half of ``gemm_os_gated``."""
+    scope (``ms_signal_set``): the producer's half of the gated calls."""
     if not (isinstance(flags, torch.Tensor) and flags.is_cuda and flags.dtype == torch.int32 and flags.dim() == 1 and flags.is_contiguous()):
         raise ValueError("flags must be a contiguous int32 GPU vector")
     if not 0 <= index < flags.numel():
@@ -252,7 +286,7 @@ def signal_set(flags: torch.Tensor, index: int, value: int = 1) -> None:
 
 
 def gate_timed_out(slice_ready: torch.Tensor) -> bool:
-    """Whether a ``gemm_os_gated`` call with these flags gave up waiting for a slice (synchronises with the device)."""
+    """Whether a gated call with these flags gave up waiting for a slice (synchronises with the device)."""
     return bool(slice_ready[-1].item() != 0)
 
 
