@@ -60,16 +60,17 @@ MS_INSTANTIATE_BIG(6, 3)
 MS_INSTANTIATE_X16(384)
 MS_INSTANTIATE_X16(256)
 #undef MS_INSTANTIATE_X16
-#define MS_INSTANTIATE_F32(WGM, WGN, T)                                                                          \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, true>(const msk::GemmArgs);     \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, false>(const msk::GemmArgs);    \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, true, true>(const msk::GemmArgs);      \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, true, true, false>(const msk::GemmArgs);     \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, true>(const msk::GemmArgs);    \
-  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, false>(const msk::GemmArgs);
-MS_INSTANTIATE_F32(4, 2, 2)
-MS_INSTANTIATE_F32(2, 2, 2)
-MS_INSTANTIATE_F32(2, 2, 1)
+#define MS_INSTANTIATE_F32(WGM, WGN, TM, TN)                                                                          \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, true, false, true>(const msk::GemmArgs);     \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, true, false, false>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, true, true, true>(const msk::GemmArgs);      \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, true, true, false>(const msk::GemmArgs);     \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, false, false, true>(const msk::GemmArgs);    \
+  template __global__ void msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, false, false, false>(const msk::GemmArgs);
+MS_INSTANTIATE_F32(4, 2, 2, 2)
+MS_INSTANTIATE_F32(4, 2, 1, 3)
+MS_INSTANTIATE_F32(2, 2, 2, 2)
+MS_INSTANTIATE_F32(2, 2, 1, 1)
 #undef MS_INSTANTIATE_F32
 
 namespace {
@@ -89,7 +90,7 @@ namespace {
 thread_local int g_variant = 0;
 thread_local int g_splits = 0;    // forced split count of the contraction (0 = library default)
 thread_local int g_launches = 0;   // kernels launched by the last GEMM call of this thread
-thread_local int g_last_variant = 0;   // bf16 kernel variant of that call's first launch (0: the fp32 kernel)
+thread_local int g_last_variant = 0;   // kernel variant of that call's first launch (bf16 tiles 1..VARIANTS, fp32 tiles F32_FIRST..F32_LAST)
 thread_local int g_last_splits = 1;    // and the number of ways it split the contraction
 thread_local int g_last_grid = 0;      // and its workgroup count
 thread_local int g_reserved_cus = 0;   // compute units the GEMM launches of this thread leave free (ms_set_reserved_cus)
@@ -314,6 +315,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 struct Pick { int v, splits; double cost; };
 
 constexpr int VARIANTS = 14;
+constexpr int F32_FIRST = 21, F32_LAST = 24;      // ids of the fp32 kernel's tiles (ms_set_variant, MS_QUERY_LAST_VARIANT)
 struct TileShape { int bm, bn; };
 constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256}, {128, 128}, {256, 256}, {256, 192},
                                              {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192},
@@ -435,7 +437,7 @@ int launch_variant(int v, int splits, const Problem &p, const DevFacts &dev, hip
 // their chunks are promised in slice order.
 int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   if (!dev.gfx950) return fail(MS_ERR_UNSUPPORTED, "the bf16 kernels need a gfx950 device");
-  if (g_variant != 0) return launch_variant(g_variant, g_splits > 1 ? g_splits : 1, p, dev, stream);
+  if (g_variant >= 1 && g_variant <= VARIANTS) return launch_variant(g_variant, g_splits > 1 ? g_splits : 1, p, dev, stream);
   const Pick single = pick_variant(p, dev);
   // (a gated product stays one launch: a second one would stand in the stream behind the first while that waits for slices)
   if (p.flow == OS && single.splits == 1 && g_splits == 0 && !p.slice_ready) {
@@ -473,11 +475,11 @@ int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   return launch_variant(single.v, single.splits, p, dev, stream);
 }
 
-// fp32 operands: gemm_f32_tile_kernel on 256 x 128 tiles (eight waves), or on 128 x 128 / 64 x 64 ones (four waves)
-// when the larger tile would leave compute units without work
-template <int WGM, int WGN, int T>
-int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
-  constexpr int BM = 32 * T * WGM, BN = 32 * T * WGN;
+// fp32 operands: gemm_f32_tile_kernel on one of its four tiles (ids F32_FIRST ..: 256 x 128 and 128 x 192 on eight
+// waves, 128 x 128 and 64 x 64 on four); `share`: two of the four-wave workgroups per compute unit
+template <int WGM, int WGN, int TM, int TN>
+int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, int id, bool share) {
+  constexpr int BM = 32 * TM * WGM, BN = 32 * TN * WGN;
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
   for (int i = 0; i < p.na; i++) g.a[i] = p.a[i];
@@ -499,39 +501,62 @@ int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   g.chunk_done = p.chunk_done;
   g.slice_ready = p.slice_ready; g.gate_ticks = p.gate_ticks;
   g_last_tiles_per_chunk = g.tiles_m * g.tiles_n;
-  // Two of the four-wave workgroups fit a compute unit (as with the 128x128 bf16 kernel, see workgroups_per_unit), but
-  // here a unit that holds two takes about 1.75 times as long over them as over one (measured: 512 tiles of 64x64 on
-  // 4096 contraction elements 0.134 ms, against 0.150 ms in two rounds of 256): sharing pays when it saves more
-  // rounds than that, otherwise the launch runs one workgroup per unit in evenly filled rounds.
-  int grid = balanced_grid(total, dev.cus);
-  if (WGM * WGN == 4 && g_reserved_cus == 0 && total > dev.cus) {
-    const long alone = (total + dev.cus - 1) / dev.cus, shared = (total + 2L * dev.cus - 1) / (2L * dev.cus);
-    if (1.75 * shared < alone) grid = total <= 2L * dev.cus ? (int)total : balanced_grid(total, 2 * dev.cus);
-  }
+  const int grid = !(share && WGM * WGN == 4) ? balanced_grid(total, dev.cus) : total <= 2L * dev.cus ? (int)total : balanced_grid(total, 2 * dev.cus);
   dim3 gd(grid), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   if (p.flow == OS) {
-    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, true><<<gd, bd, 0, stream>>>(g);
-    else msk::gemm_f32_tile_kernel<WGM, WGN, T, true, false, false><<<gd, bd, 0, stream>>>(g);
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, true, false, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, true, false, false><<<gd, bd, 0, stream>>>(g);
   } else if (p.flow == LS) {
-    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, T, true, true, true><<<gd, bd, 0, stream>>>(g);
-    else msk::gemm_f32_tile_kernel<WGM, WGN, T, true, true, false><<<gd, bd, 0, stream>>>(g);
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, true, true, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, true, true, false><<<gd, bd, 0, stream>>>(g);
   } else {
-    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, true><<<gd, bd, 0, stream>>>(g);
-    else msk::gemm_f32_tile_kernel<WGM, WGN, T, false, false, false><<<gd, bd, 0, stream>>>(g);
+    if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, false, false, true><<<gd, bd, 0, stream>>>(g);
+    else msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, false, false, false><<<gd, bd, 0, stream>>>(g);
   }
-  if (g_launches == 0) g_last_grid = (int)gd.x;
+  if (g_launches == 0) { g_last_grid = (int)gd.x; g_last_variant = id; }
   g_launches++;
   MS_HIP(hipGetLastError());
   return MS_OK;
 }
 
+// The fp32 tiles as the chooser prices them: time per output element and contraction step relative to the 256 x 128
+// tile's, for a unit that holds one workgroup, and the factor by which a unit that holds two four-wave workgroups takes
+// longer over the pair.  Fitted to ten products from 512^2 x 1024 to 4096^3 (one round of 256 tiles of 128 x 192 on
+// 4096 contraction elements 363 us, of 256 x 128 468 us, of 128 x 128 on 8192 elements 510 us; 512 tiles of 64 x 64
+// shared 133 us, alone in two rounds 150 us; 1024 tiles of 128 x 128 shared 957 us).  Unlike the bf16 kernels this one
+// does not sit on the power limit: a partly filled round costs a whole one.
+struct F32Tile { int id, bm, bn; bool four_waves; double cost, shared; };
+constexpr F32Tile F32_TILES[] = {{F32_FIRST, 256, 128, false, 1.0, 0.0}, {F32_FIRST + 1, 128, 192, false, 1.0 / 0.967, 0.0},
+                                 {F32_FIRST + 2, 128, 128, true, 1.0 / 0.918, 1.88}, {F32_FIRST + 3, 64, 64, true, 1.0 / 0.78, 1.78}};
+
+int launch_f32_id(int id, bool share, const Problem &p, const DevFacts &dev, hipStream_t stream) {
+  switch (id) {
+    case F32_FIRST: return launch_f32_tile<4, 2, 2, 2>(p, dev, stream, id, false);
+    case F32_FIRST + 1: return launch_f32_tile<4, 2, 1, 3>(p, dev, stream, id, false);
+    case F32_FIRST + 2: return launch_f32_tile<2, 2, 2, 2>(p, dev, stream, id, share);
+    default: return launch_f32_tile<2, 2, 1, 1>(p, dev, stream, id, share);
+  }
+}
+
 int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   const long chunks = p.flow == OS ? 1 : p.S;
-  const long big = (long)((p.M + 255) / 256) * ((p.N + 127) / 128) * chunks;
-  const long mid = (long)((p.M + 127) / 128) * ((p.N + 127) / 128) * chunks;
-  if (big >= dev.cus) return launch_f32_tile<4, 2, 2>(p, dev, stream);
-  return mid >= dev.cus ? launch_f32_tile<2, 2, 2>(p, dev, stream) : launch_f32_tile<2, 2, 1>(p, dev, stream);
+  int best = 0;
+  bool best_share = false;
+  double best_cost = 0.0;
+  for (const F32Tile &t : F32_TILES) {
+    if (g_variant >= F32_FIRST && g_variant != t.id) continue;
+    const long tiles = (long)((p.M + t.bm - 1) / t.bm) * ((p.N + t.bn - 1) / t.bn) * chunks;
+    const double area = (double)t.bm * t.bn * t.cost;
+    double cost = (double)((tiles + dev.cus - 1) / dev.cus) * area;
+    bool share = false;
+    if (t.four_waves && g_reserved_cus == 0 && tiles > dev.cus) {
+      const double both = (double)((tiles + 2L * dev.cus - 1) / (2L * dev.cus)) * area * t.shared;
+      if (both < cost) { cost = both; share = true; }
+    }
+    if (best == 0 || cost < best_cost) { best = t.id; best_cost = cost; best_share = share; }
+  }
+  return launch_f32_id(best, best_share, p, dev, stream);
 }
 
 // the device as this thread's launches may use it: without the compute units it has been told to leave free
@@ -629,7 +654,8 @@ MS_API long ms_query(int what) {
 
 MS_API int ms_set_variant(int variant) {
   const int v = variant % 100, splits = variant / 100;
-  if (variant < 0 || v > VARIANTS || splits == 1 || splits > SPLIT_MAX) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  const bool f32_tile = variant >= F32_FIRST && variant <= F32_LAST;      // (never split)
+  if (variant < 0 || (!f32_tile && (v > VARIANTS || splits == 1 || splits > SPLIT_MAX))) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
   g_variant = v;
   g_splits = splits;
   return MS_OK;
@@ -772,7 +798,7 @@ MS_API int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_
   // what the library would do with room to spare decides whether the built-in scratch is needed, and whether it is enough
   p.ws = reinterpret_cast<void *>(uintptr_t(256));    // stands for "a workspace": only its size is looked at here
   p.ws_bytes = ~size_t(0);
-  const Pick want = g_variant != 0 ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, usable(*dev));
+  const Pick want = g_variant >= 1 && g_variant <= VARIANTS ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, usable(*dev));
   if (want.splits <= 1) {
     // an unsplit product exchanges nothing (without a workspace the library makes the same choice: splits are only ever added)
     p.ws = nullptr;

@@ -65,6 +65,32 @@ def test_default_choice_is_close_to_the_best_variant(flow, shape):
         f"variant {best_v} {times[best_v] * 1e6:.0f} us; all: " + " ".join(f"{v}:{t * 1e6:.0f}" for v, t in times.items()))
 
 
+@pytest.mark.parametrize("shape", [(2048, 3072, 2048), (3072, 3072, 2048), (2048, 6144, 1024), (4096, 4096, 1024), (2048, 2048, 4096), (1024, 2048, 2048),
+                                   (1536, 1536, 2048)], ids=lambda s: "x".join(map(str, s)))
+def test_fp32_default_tile_is_close_to_the_best_tile(shape):
+    """The fp32 kernel's tile choice (rounds x tile area x fitted cost) against each of its four tiles forced."""
+    lib = _lib.load()
+    m, n, k = shape
+    g = torch.Generator(device="cuda").manual_seed(3)
+    A = torch.randn((m, k), generator=g, device="cuda"); B = torch.randn((k, n), generator=g, device="cuda")
+    C = torch.empty((m, n), device="cuda")
+    import meshslice_amd as ms
+    run = lambda: ms.gemm_os([A], [B], out=C)
+    times = {}
+    try:
+        for rnd in range(2):
+            for v in (0, 21, 22, 23, 24):
+                assert lib.ms_set_variant(v) == 0
+                t = _sustained(run)
+                times[v] = min(times.get(v, t), t)
+                if v == 0:
+                    picked = int(lib.ms_query(_lib.MS_QUERY_LAST_VARIANT))
+    finally:
+        lib.ms_set_variant(0)
+    best = min((21, 22, 23, 24), key=lambda v: times[v])
+    assert times[0] <= SLACK * times[best], f"default (tile {picked}) {times[0] * 1e6:.0f} us; " + " ".join(f"{v}:{t * 1e6:.0f}" for v, t in times.items())
+
+
 @pytest.mark.parametrize("flow", ["ls", "rs"])
 def test_a_watcher_sees_chunks_complete_before_the_kernel_ends(flow):
     S, m, n, k, BAND = 8, 8192, 1536, 8192, 48      # about 1.3 ms of kernel: room for some tens of polls
