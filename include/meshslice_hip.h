@@ -107,8 +107,8 @@ int ms_gemm_os_fused(const void *const *A_slices, const void *const *B_slices, i
  * K range of every tile into 2..8 parts that run on different compute units; each part leaves its fp32 partial tile in
  * the workspace, and the part that finishes last adds them up in a fixed order (so the result does not depend on
  * timing: the same call gives the same bits every time) and writes its part of C.  Only the plain product is split: with
- * an activation, a residual or row moments the call runs as ms_gemm_os_fused does.  No counterpart in the reference, where
- * XLA picks the contraction's schedule.
+ * an activation, a residual or row moments the call runs as ms_gemm_os_fused does.  bf16 and fp32 products split alike.
+ * No counterpart in the reference, where XLA picks the contraction's schedule.
  * workspace: device memory, 256-byte aligned, prepared once with ms_workspace_init and then reusable by any number of
  * calls, one at a time (calls that share a workspace must not overlap: same stream, or ordered by events);
  * ms_workspace_bytes() is the size with which no product is refused a split for lack of room, a smaller one only
@@ -125,7 +125,8 @@ int ms_gemm_os_ws(const void *const *A_slices, const void *const *B_slices, int 
  * split-contraction workspace is a fixed array inside the library's code object (4096 + 48 MiB per device, held until the
  * process ends); the call allocates and frees nothing.  A product whose exchange of partial tiles would not fit that
  * array is refused with MS_ERR_UNSUPPORTED (the message names the sizes) — use ms_gemm_os_ws there.  Only products that
- * split their contraction touch the array (few output tiles, a long contraction); all such calls on one device share it.
+ * split their contraction touch the array (few output tiles, a long contraction; bf16 operands only: an fp32 product
+ * runs unsplit here); all such calls on one device share it.
  * Calls on one stream are ordered by the stream.  A call that arrives on another stream than the array's previous user
  * first waits for the device to go idle (hipDeviceSynchronize, under a per-device lock held until the call's kernels
  * are queued), so eager calls from several streams or host threads never meet in the array — at the price of that wait
@@ -341,7 +342,7 @@ int ms_probe_l2_lds_stream(const void *buffer, size_t buffer_bytes, int region_s
 /* Hook for tests and measurements (thread-local): later bf16 calls on this thread use tile variant `variant % 100`
  * (1..14, 0 = the library's choice) and split the contraction `variant / 100` ways (2..8, 0 = the library's choice;
  * a forced split needs a workspace and an output-stationary product).  21..24 name the fp32 kernel's tiles instead
- * (256x128, 128x192, 128x128, 64x64; never split): fp32 calls then use that tile and bf16 calls the library's choice,
+ * (256x128, 128x192, 128x128, 64x64; split counts as above): fp32 calls then use that tile and bf16 calls the library's choice,
  * as fp32 calls do under 1..14.  Unknown ids are rejected with MS_ERR_ARG. */
 int ms_set_variant(int variant);
 

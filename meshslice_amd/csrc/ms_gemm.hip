@@ -477,8 +477,10 @@ int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
 
 // fp32 operands: gemm_f32_tile_kernel on one of its four tiles (ids F32_FIRST ..: 256 x 128 and 128 x 192 on eight
 // waves, 128 x 128 and 64 x 64 on four); `share`: two of the four-wave workgroups per compute unit
+int f32_split_refused(const Problem &p, const DevFacts &dev, int bm, int bn, int splits);
+
 template <int WGM, int WGN, int TM, int TN>
-int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, int id, bool share) {
+int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, int id, bool share, int splits) {
   constexpr int BM = 32 * TM * WGM, BN = 32 * TN * WGN;
   msk::GemmArgs g;
   memset(&g, 0, sizeof(g));
@@ -501,7 +503,15 @@ int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, i
   g.chunk_done = p.chunk_done;
   g.slice_ready = p.slice_ready; g.gate_ticks = p.gate_ticks;
   g_last_tiles_per_chunk = g.tiles_m * g.tiles_n;
-  const int grid = !(share && WGM * WGN == 4) ? balanced_grid(total, dev.cus) : total <= 2L * dev.cus ? (int)total : balanced_grid(total, 2 * dev.cus);
+  if (splits > 1) {
+    const int why = f32_split_refused(p, dev, BM, BN, splits);
+    if (why) return fail(MS_ERR_ARG, "contraction cannot be split %d ways here: %s", splits, SPLIT_REFUSALS[why]);
+    g.splits = splits;
+    g.ws_count = static_cast<int *>(p.ws);
+    g.ws_tiles = static_cast<char *>(p.ws) + WS_HEADER_BYTES;
+  }
+  const long items = total * g.splits;
+  const int grid = !(share && WGM * WGN == 4) ? balanced_grid(items, dev.cus) : items <= 2L * dev.cus ? (int)items : balanced_grid(items, 2 * dev.cus);
   dim3 gd(grid), bd(WGM * WGN * 64);
   const bool obf = p.out_dtype == MS_DTYPE_BF16;
   if (p.flow == OS) {
@@ -514,10 +524,23 @@ int launch_f32_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, i
     if (obf) msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, false, false, true><<<gd, bd, 0, stream>>>(g);
     else msk::gemm_f32_tile_kernel<WGM, WGN, TM, TN, false, false, false><<<gd, bd, 0, stream>>>(g);
   }
-  if (g_launches == 0) { g_last_grid = (int)gd.x; g_last_variant = id; }
+  if (g_launches == 0) { g_last_grid = (int)gd.x; g_last_variant = id; g_last_splits = g.splits; }
   g_launches++;
   MS_HIP(hipGetLastError());
   return MS_OK;
+}
+
+// 0 if the fp32 product p can run on a bm x bn tile with its contraction split `splits` ways, else an index into SPLIT_REFUSALS
+int f32_split_refused(const Problem &p, const DevFacts &dev, int bm, int bn, int splits) {
+  if (splits < 2 || splits > SPLIT_MAX) return 7;
+  if (p.flow != OS) return 1;
+  if (!p.ws) return 2;
+  const long tiles = (long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
+  if (tiles * splits > dev.cus) return 3;
+  if (tiles > WS_MAX_TILES) return 4;
+  if ((size_t)(tiles * splits) * bm * bn * sizeof(float) + WS_HEADER_BYTES > p.ws_bytes) return 5;
+  if (((long)(p.K + 31) / 32) * p.S < splits) return 6;     // every part needs at least one K step
+  return 0;
 }
 
 // The fp32 tiles as the chooser prices them: time per output element and contraction step relative to the 256 x 128
@@ -530,33 +553,52 @@ struct F32Tile { int id, bm, bn; bool four_waves; double cost, shared; };
 constexpr F32Tile F32_TILES[] = {{F32_FIRST, 256, 128, false, 1.0, 0.0}, {F32_FIRST + 1, 128, 192, false, 1.0 / 0.967, 0.0},
                                  {F32_FIRST + 2, 128, 128, true, 1.0 / 0.918, 1.88}, {F32_FIRST + 3, 64, 64, true, 1.0 / 0.78, 1.78}};
 
-int launch_f32_id(int id, bool share, const Problem &p, const DevFacts &dev, hipStream_t stream) {
+int launch_f32_id(int id, bool share, int splits, const Problem &p, const DevFacts &dev, hipStream_t stream) {
   switch (id) {
-    case F32_FIRST: return launch_f32_tile<4, 2, 2, 2>(p, dev, stream, id, false);
-    case F32_FIRST + 1: return launch_f32_tile<4, 2, 1, 3>(p, dev, stream, id, false);
-    case F32_FIRST + 2: return launch_f32_tile<2, 2, 2, 2>(p, dev, stream, id, share);
-    default: return launch_f32_tile<2, 2, 1, 1>(p, dev, stream, id, share);
+    case F32_FIRST: return launch_f32_tile<4, 2, 2, 2>(p, dev, stream, id, false, splits);
+    case F32_FIRST + 1: return launch_f32_tile<4, 2, 1, 3>(p, dev, stream, id, false, splits);
+    case F32_FIRST + 2: return launch_f32_tile<2, 2, 2, 2>(p, dev, stream, id, share, splits);
+    default: return launch_f32_tile<2, 2, 1, 1>(p, dev, stream, id, share, splits);
   }
 }
 
+// An output-stationary fp32 product whose tiles leave compute units idle may split its contraction like the bf16 ones
+// (work items = tiles x splits, see split_k_exchange).  The exchange of the partial tiles is priced, in the chooser's
+// unit (the 256 x 128 tile's time per output element and contraction step, 3.5e-6 us), at
+// (F32_SPLIT_FIX + splits x m x n x F32_SPLIT_PER_ELEMENT) / K: about 5 us plus 2 us per million partial elements,
+// fitted to 2048 x 2048 x 8192 (128 tiles of 256 x 128 in two parts: 484 us against 513 us unsplit on 128 x 128) and
+// 1536 x 1536 x 4096 (72 tiles in three parts: 179 us against 224 us on 64 x 64 tiles in three rounds).
+constexpr double F32_SPLIT_FIX = 1.43e6, F32_SPLIT_PER_ELEMENT = 0.6;
+constexpr long F32_SPLIT_MIN_K = 256;      // contraction elements per split item, at least
+
 int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   const long chunks = p.flow == OS ? 1 : p.S;
-  int best = 0;
+  const long total_k = (long)p.K * (p.flow == OS ? p.S : 1);
+  const bool forced_tile = g_variant >= F32_FIRST;
+  int best = 0, best_splits = 1;
   bool best_share = false;
   double best_cost = 0.0;
   for (const F32Tile &t : F32_TILES) {
-    if (g_variant >= F32_FIRST && g_variant != t.id) continue;
+    if (forced_tile && g_variant != t.id) continue;
     const long tiles = (long)((p.M + t.bm - 1) / t.bm) * ((p.N + t.bn - 1) / t.bn) * chunks;
     const double area = (double)t.bm * t.bn * t.cost;
-    double cost = (double)((tiles + dev.cus - 1) / dev.cus) * area;
-    bool share = false;
-    if (t.four_waves && g_reserved_cus == 0 && tiles > dev.cus) {
-      const double both = (double)((tiles + 2L * dev.cus - 1) / (2L * dev.cus)) * area * t.shared;
-      if (both < cost) { cost = both; share = true; }
+    for (int splits = 1; splits <= SPLIT_MAX; splits++) {
+      if (forced_tile && g_splits != 0 && splits != g_splits) continue;
+      if (!forced_tile && g_splits != 0) { if (splits > 1) break; }      // (a split forced for the bf16 tiles says nothing here)
+      if (splits > 1 && (f32_split_refused(p, dev, t.bm, t.bn, splits) || (!(forced_tile && g_splits != 0) && total_k / splits < F32_SPLIT_MIN_K))) continue;
+      const long items = tiles * splits;
+      double cost = (double)((items + dev.cus - 1) / dev.cus) * area / splits;
+      bool share = false;
+      if (t.four_waves && g_reserved_cus == 0 && items > dev.cus) {
+        const double both = (double)((items + 2L * dev.cus - 1) / (2L * dev.cus)) * area * t.shared / splits;
+        if (both < cost) { cost = both; share = true; }
+      }
+      if (splits > 1) cost += (F32_SPLIT_FIX + (double)splits * p.M * p.N * F32_SPLIT_PER_ELEMENT) / total_k;
+      if (best == 0 || cost < best_cost) { best = t.id; best_cost = cost; best_share = share; best_splits = splits; }
     }
-    if (best == 0 || cost < best_cost) { best = t.id; best_cost = cost; best_share = share; }
   }
-  return launch_f32_id(best, best_share, p, dev, stream);
+  if (best == 0) return fail(MS_ERR_ARG, "contraction cannot be split %d ways on fp32 tile %d here", g_splits, g_variant);
+  return launch_f32_id(best, best_share, best_splits, p, dev, stream);
 }
 
 // the device as this thread's launches may use it: without the compute units it has been told to leave free
@@ -654,8 +696,8 @@ MS_API long ms_query(int what) {
 
 MS_API int ms_set_variant(int variant) {
   const int v = variant % 100, splits = variant / 100;
-  const bool f32_tile = variant >= F32_FIRST && variant <= F32_LAST;      // (never split)
-  if (variant < 0 || (!f32_tile && (v > VARIANTS || splits == 1 || splits > SPLIT_MAX))) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
+  const bool known = v <= VARIANTS || (v >= F32_FIRST && v <= F32_LAST);
+  if (variant < 0 || !known || splits == 1 || splits > SPLIT_MAX) return fail(MS_ERR_ARG, "ms_set_variant: unknown variant %d", variant);
   g_variant = v;
   g_splits = splits;
   return MS_OK;
@@ -791,7 +833,7 @@ MS_API int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_
   Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
   int rc = validate(p);
   if (rc) return rc;
-  if (in_dtype != MS_DTYPE_BF16) return run(p, stream);     // the fp32 kernels never split: no scratch
+  if (in_dtype != MS_DTYPE_BF16) return run(p, stream);     // without a workspace an fp32 product is never split: no scratch
   DevInfo *dev = nullptr;
   rc = dev_info(&dev);
   if (rc) return rc;

@@ -387,7 +387,7 @@ def test_c_abi_rejects_bad_arguments():
     null, _k3 = _lib.ptr_array([0])
     assert call(pa=null) == _lib.MS_ERR_ARG
     assert lib.ms_set_variant(99) == _lib.MS_ERR_ARG
-    assert lib.ms_set_variant(25) == _lib.MS_ERR_ARG and lib.ms_set_variant(221) == _lib.MS_ERR_ARG      # fp32 tiles are 21-24 and never split
+    assert lib.ms_set_variant(25) == _lib.MS_ERR_ARG and lib.ms_set_variant(121) == _lib.MS_ERR_ARG      # fp32 tiles are 21-24; a split is 2..8 ways
     with pytest.raises(ValueError):
         ms.gemm_os([a], [torch.zeros((32, 64), dtype=torch.bfloat16, device="cuda")])
     with pytest.raises(ValueError):

@@ -64,6 +64,69 @@ def test_forced_split_matches_oracle_and_is_bit_reproducible(variant, splits):
     assert torch.equal(out_bf16, got.to(torch.bfloat16))        # bf16 output = one rounding of the same sums
 
 
+def _unsplit(A, B, out_dtype=torch.float32):
+    """The same product through ms_gemm_os, which has no workspace and therefore never splits."""
+    L = _lib.load()
+    S, (m, ks), n = len(A), A[0].shape, B[0].shape[1]
+    pa, _ka = _lib.ptr_array([t.data_ptr() for t in A]); pb, _kb = _lib.ptr_array([t.data_ptr() for t in B])
+    C = torch.empty((m, n), dtype=out_dtype, device="cuda")
+    dt = _lib.MS_DTYPE_BF16 if A[0].dtype == torch.bfloat16 else _lib.MS_DTYPE_F32
+    rc = L.ms_gemm_os(pa, pb, S, m, n, ks, ks, n, ctypes.c_void_p(C.data_ptr()), n, dt,
+                      _lib.MS_DTYPE_BF16 if out_dtype == torch.bfloat16 else _lib.MS_DTYPE_F32, None)
+    assert rc == 0 and L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+    return C
+
+
+@pytest.mark.parametrize("tile", [21, 22, 23, 24])
+@pytest.mark.parametrize("splits", [2, 3, 8])
+def test_fp32_forced_split_matches_oracle_and_is_bit_reproducible(tile, splits):
+    """The fp32 kernel's split contraction on each of its tiles: ragged edges, a K tail, K steps that do not divide by the
+    split count, slices that a split's K range crosses.  Tolerance 1e-5 of the result's norm (fp32 in and out)."""
+    L = _lib.load()
+    m, n, ks, S = 200, 424, 708, 3             # 3 slices of 708 = 22.1 K steps of 32 each
+    g = torch.Generator(device="cuda").manual_seed(100 * tile + splits)
+    A = [torch.randn((m, ks), generator=g, device="cuda") for _ in range(S)]
+    B = [torch.randn((ks, n), generator=g, device="cuda") * 0.05 for _ in range(S)]
+    want = sum(_f64(a) @ _f64(b) for a, b in zip(A, B))
+    L.ms_set_variant(tile)
+    plain = _unsplit(A, B)
+    assert L.ms_query(_lib.MS_QUERY_LAST_VARIANT) == tile
+    L.ms_set_variant(tile + 100 * splits)
+    got = ms.gemm_os(A, B)
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == splits and L.ms_query(_lib.MS_QUERY_LAST_VARIANT) == tile
+    assert orc.rel_frobenius(_f64(got), want) <= 1e-5
+    assert orc.rel_frobenius(_f64(got), _f64(plain)) <= 1e-6
+    for _ in range(3):
+        assert torch.equal(ms.gemm_os(A, B), got)
+    torch.cuda.synchronize()
+    assert int(_counters().abs().sum()) == 0
+    assert torch.equal(ms.gemm_os(A, B, out_dtype=torch.bfloat16), got.to(torch.bfloat16))
+
+
+def test_fp32_product_of_well_under_one_round_is_split_by_default():
+    """1536 x 1536 x 4096 in fp32: 72 tiles of 256x128 (or 576 of 64x64 in three rounds) for 256 compute units."""
+    L = _lib.load()
+    g = torch.Generator(device="cuda").manual_seed(5)
+    A = [torch.randn((1536, 2048), generator=g, device="cuda") for _ in range(2)]
+    B = [torch.randn((2048, 1536), generator=g, device="cuda") * 0.02 for _ in range(2)]
+    C = ms.gemm_os(A, B)
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) > 1 and 21 <= L.ms_query(_lib.MS_QUERY_LAST_VARIANT) <= 24
+    rows = np.random.default_rng(0).choice(1536, 64, replace=False)
+    want = sum(_f64(a[rows]) @ _f64(b) for a, b in zip(A, B))
+    assert orc.rel_frobenius(_f64(C[rows]), want) <= 1e-5
+    assert torch.equal(ms.gemm_os(A, B), C)
+    assert orc.rel_frobenius(_f64(_unsplit(A, B)), _f64(C)) <= 1e-6
+    # LS / RS chunks and products with a tile per unit stay unsplit
+    ms.gemm_ls(A[0], [B[0].t().contiguous()])
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+    ms.gemm_os([torch.randn((4096, 256), generator=g, device="cuda")], [torch.randn((256, 4096), generator=g, device="cuda")])
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
+    # a forced split that cannot be: more items than compute units
+    L.ms_set_variant(824)
+    with pytest.raises(ValueError, match="cannot be split"):
+        ms.gemm_os(A, B)
+
+
 def test_small_output_long_contraction_is_split_by_default():
     """2048 x 1536 x 12288 (out_proj backward-data on an 8x8 mesh): 64 tiles for 256 compute units."""
     L = _lib.load()
