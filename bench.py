@@ -29,7 +29,7 @@ PEAK_FP32_TFLOPS = 157.3      # MI355X dense fp32 MFMA
 # HBM-side traffic per config-2 launch from rocprofv3 (FETCH_SIZE x the factor a 1 GiB copy gives in the same run + WRITE_SIZE),
 # per kernel variant: a figure measured offline on that kernel, reported only when the run used it
 TRAFFIC_PROFILES = {
-    12: {"bytes": int(round(688312.0 * 1024 * 1048576 / 524314.0 + 98428.6 * 1024)),
+    12: {"bytes": int(round(688301.0 * 1024 * 1048576 / 524314.0 + 98447.1 * 1024)),
          "source": "profiles/gemm_bf16_x16_256x384x64_os_cfg2.md @ variant 12 (gemm_bf16_x16_kernel, 256x384x64 tile)"},
     10: {"bytes": int(round(698639.1 * 1024 * 1048576 / 524313.19 + 114688 * 1024)),
          "source": "profiles/gemm_bf16_big_256x384x64_os_cfg2.md @ variant 10 (gemm_bf16_big_kernel<4,6>, 256x384x64 tile)"},
