@@ -4,7 +4,10 @@
 * the library's default tile choice is within 15 % of the best forced variant's time on products outside the GPT-3
   family (shapes and operands of tests/test_gpu_chooser.py, whose own test checks the results);
 * a watcher on a second stream sees chunks of a counted LS / RS call complete before the kernel has ended
-  (tests/test_gpu_signal.py checks that what it then reads is the finished chunk).
+  (tests/test_gpu_signal.py checks that what it then reads is the finished chunk);
+* one gated and counted LS / RS launch, its slices arriving 150 us apart on a producer stream, has chunk 0 complete
+  before the last slice has been flagged (tests/test_zx_gpu_gate.py checks the results of such calls);
+* the fp32 kernel's tile choice is within 15 % of the best of its four tiles forced.
 
 Times are sustained wall-clock means (warm-up, then a loop between two synchronisations), the best of two rounds per
 candidate, so that one host hiccup does not decide the comparison.  Marked ``perf`` besides ``gpu``:
@@ -103,3 +106,67 @@ def test_a_watcher_sees_chunks_complete_before_the_kernel_ends(flow):
         if early and len(h) > 2:
             break
     assert early, "no chunk was seen complete before the kernel had ended"
+
+
+@pytest.mark.parametrize("flow", ["ls", "rs"])
+def test_one_launch_with_both_ends_open_hands_on_chunk_0_before_the_last_slice_has_arrived(flow):
+    """ms_gemm_ls_gated / ms_gemm_rs_gated with completion counters: the product is enqueued first, a producer stream
+    then delivers slice after slice about 150 us apart (a copy, a delay, the flag), and a watcher polls flags and
+    counters from the host.  Chunk 0 must be seen complete while the last flag is still down: the launch multiplies what
+    has arrived while the rest is on its way, and says which chunks may already be handed on."""
+    import meshslice_amd as ms
+    S, m, n, k = 8, 8192, 1536, 8192
+    lib = _lib.load()
+    src = signal_tests._operands(flow, m, n, k, S, torch.bfloat16)
+    which = 1 if flow == "ls" else 0
+    ops = list(src)
+    ops[which] = [torch.zeros_like(t) for t in src[which]]
+    gated = ms.gemm_ls_gated if flow == "ls" else ms.gemm_rs_gated
+    ready = torch.zeros(S + 1, dtype=torch.int32, device="cuda")
+    done = torch.zeros(S, dtype=torch.int32, device="cuda")
+    seen_ready = torch.zeros(S + 1, dtype=torch.int32).pin_memory()
+    seen_done = torch.zeros(S, dtype=torch.int32).pin_memory()
+    compute, producer, watch = torch.cuda.Stream(), torch.cuda.Stream(), torch.cuda.Stream()
+    try:
+        assert lib.ms_set_reserved_cus(32) == 0        # the producer's copies and the watcher's need compute units beside the product
+        want = signal_tests._plain(flow, src, torch.bfloat16)
+    finally:
+        lib.ms_set_reserved_cus(0)
+    early = []
+    for attempt in range(4):          # the first call also loads code and sets up the streams: it may be over before the first poll
+        for t in ops[which]:
+            t.zero_()
+        ready.zero_(); done.zero_()
+        torch.cuda.synchronize()
+        try:
+            assert lib.ms_set_reserved_cus(32) == 0
+            with torch.cuda.stream(compute):
+                got, tiles = gated(*ops, ready, out_dtype=torch.bfloat16, chunk_done=done, timeout_ms=1500)
+        finally:
+            lib.ms_set_reserved_cus(0)
+        with torch.cuda.stream(producer):
+            for s_ in range(S):
+                ops[which][s_].copy_(src[which][s_])
+                torch.cuda._sleep(300000)                   # about 150 us
+                ms.signal_set(ready, s_)
+        history = []
+        with torch.cuda.stream(watch):
+            for poll in range(2000):                        # bounded: the watcher gives up, it never waits for the kernel
+                seen_ready.copy_(ready, non_blocking=True)  # (flags first: a chunk seen complete after a flag seen down was complete before the flag went up)
+                seen_done.copy_(done, non_blocking=True)
+                watch.synchronize()
+                history.append((seen_ready.tolist(), seen_done.tolist()))
+                if history[-1][1] == [tiles] * S or history[-1][0][S]:
+                    break
+        torch.cuda.synchronize()
+        if ms.gate_timed_out(ready):
+            pytest.skip("the producer's copies did not run beside the waiting product on this machine")
+        assert done.tolist() == [tiles] * S
+        for s_ in range(S):
+            assert torch.equal(got[s_], want[s_])
+        early = [i for i, (r, d) in enumerate(history) if d[0] == tiles and r[S - 1] == 0]
+        if early:
+            break
+    assert early, f"chunk 0 was never seen complete while the last flag was down ({len(history)} polls)"
+    first = history[early[0]]
+    print(f"\n{flow}: {len(history)} polls; chunk 0 first seen complete with {sum(first[0][:S])} of {S} slices flagged and {sum(d == tiles for d in first[1])} chunks complete")
