@@ -1,4 +1,4 @@
-"""Two yardsticks for the tile chooser and the kernels behind it, on products outside the GPT-3 family.
+"""Yardsticks for the tile choosers and the kernels behind them, on products outside the GPT-3 family.
 
 ``python3 -m meshslice_amd.compare vendor [--small]``
     this build's one-slice bf16 product (bf16 in and out) beside the vendor library's (``torch.matmul``) for the three
@@ -8,6 +8,11 @@
 ``python3 -m meshslice_amd.compare chooser [--cases N] [--slices S] [--seed K]``
     how far the default tile choice is from the best of ten forced tile variants, on N shapes drawn at random per
     dataflow (dimensions 512..16384, 0.02..3 TFLOP per product), S slices each.
+
+``python3 -m meshslice_amd.compare fp32``
+    the fp32 kernel's default choice (tile and split count), each of its four tiles forced (ids 21..24, each with the
+    split count the library would take for it) and the vendor library's product, output-stationary, on ten products
+    from 512 x 512 x 1024 to 4096^3.
 
 Every time is the mean of back-to-back launches between two HIP events after warm-up launches (a launch timed alone,
 the device idling before it, reads 3-15 % longer); one line per case, then a JSON summary.  The measurement protocol
@@ -130,15 +135,54 @@ def chooser(cases, S, seed):
     return out
 
 
+FP32_SHAPES = [(4096, 4096, 4096), (8192, 2048, 2048), (3072, 3072, 4096), (2048, 3072, 4096), (2048, 6144, 2048), (2048, 2048, 8192),
+               (1536, 1536, 4096), (1024, 2048, 4096), (1024, 1024, 1024), (512, 512, 1024)]
+FP32_TILES = (21, 22, 23, 24)      # 256x128, 128x192 (eight waves), 128x128, 64x64 (four waves)
+
+
+def fp32(shapes=FP32_SHAPES):
+    lib = _lib.load()
+    _settle()
+    ratios, off = [], []
+    for (m, n, k) in shapes:
+        g = torch.Generator(device="cuda").manual_seed(m + n + k)
+        A = torch.randn((m, k), generator=g, device="cuda"); B = torch.randn((k, n), generator=g, device="cuda") * 0.02
+        C = torch.empty((m, n), device="cuda")
+        ours = lambda: gemm_os([A], [B], out=C)
+        theirs = lambda: torch.matmul(A, B, out=C)
+        times, what = {}, {}
+        try:
+            for _ in range(2):
+                for v in (0,) + FP32_TILES:
+                    lib.ms_set_variant(v)
+                    t = _sustained_us(ours, 15, 40)
+                    times[v] = min(times.get(v, t), t)
+                    what[v] = (int(lib.ms_query(_lib.MS_QUERY_LAST_VARIANT)), int(lib.ms_query(_lib.MS_QUERY_LAST_SPLITS)))
+                lib.ms_set_variant(0)
+                tv = _sustained_us(theirs, 15, 40)
+                times["vendor"] = min(times.get("vendor", tv), tv)
+        finally:
+            lib.ms_set_variant(0)
+        best = min(FP32_TILES, key=lambda v: times[v])
+        fl = 2.0 * m * n * k
+        ratios.append(times["vendor"] / times[0]); off.append(times[0] / times[best])
+        print(f"fp32 {m}x{n}x{k}: default tile {what[0][0]} x{what[0][1]} {times[0]:.0f} us {fl / times[0] / 1e6:.1f} TFLOP/s | forced "
+              + " ".join(f"{v}(x{what[v][1]}):{times[v]:.0f}" for v in FP32_TILES) + f" | vendor {times['vendor']:.0f} us | vendor time / this build's "
+              f"{times['vendor'] / times[0]:.3f}", flush=True)
+    return {"cases": len(ratios), "vendor_over_ours_geometric_mean": round(statistics.geometric_mean(ratios), 3), "min": round(min(ratios), 3),
+            "max": round(max(ratios), 3), "default_over_best_tile_max": round(max(off), 3)}
+
+
 def main(argv=None) -> None:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     sub = ap.add_subparsers(dest="what", required=True)
     pv = sub.add_parser("vendor"); pv.add_argument("--small", action="store_true")
     pc = sub.add_parser("chooser")
+    sub.add_parser("fp32")
     pc.add_argument("--cases", type=int, default=60); pc.add_argument("--slices", type=int, default=2); pc.add_argument("--seed", type=int, default=5)
     args = ap.parse_args(argv)
     torch.cuda.set_device(0)
-    res = vendor(SMALL if args.small else LARGE) if args.what == "vendor" else chooser(args.cases, args.slices, args.seed)
+    res = vendor(SMALL if args.small else LARGE) if args.what == "vendor" else fp32() if args.what == "fp32" else chooser(args.cases, args.slices, args.seed)
     print(json.dumps({args.what: res}), flush=True)
 
 

@@ -85,10 +85,12 @@ def test_l2_lds_stream_probe_reports_a_rate_inside_the_machines_limits():
 
 def test_the_comparison_tool_times_a_small_product_both_ways():
     """``python3 -m meshslice_amd.compare``: one small product beside the vendor library's in all three layouts, and the
-    default tile choice against the forced variants on one random shape per dataflow."""
+    default tile choice against the forced variants on one random shape per dataflow; the fp32 kernel's tiles on one small product."""
     from meshslice_amd import compare
     res = compare.vendor([(1024, 1024, 1024)])
     assert set(res) == {"nn", "nt", "tn"} and all(r["cases"] == 1 and 0.2 < r["geometric_mean"] < 5.0 for r in res.values())
     res = compare.chooser(1, 2, 3)
     assert set(res) == {"os", "ls", "rs"} and all(r["cases"] == 1 and 0.5 < r["max"] < 1.5 for r in res.values())
     assert _lib.load().ms_query(_lib.MS_QUERY_LAST_VARIANT) >= 1
+    res = compare.fp32([(1024, 1024, 512)])
+    assert res["cases"] == 1 and 0.2 < res["vendor_over_ours_geometric_mean"] < 5.0 and res["default_over_best_tile_max"] < 1.5
