@@ -55,7 +55,7 @@ extern "C" {
                                    would leave much of the last round of compute units idle is done in two launches) */
 #define MS_QUERY_LAST_SPLITS 7   /* ways in which that launch split the contraction (1: not split) */
 #define MS_QUERY_LAST_VARIANT 6  /* kernel variant (tile shape, see ms_set_variant) of the first of those launches: 1..14 for
-                                   the bf16 kernels, 21..24 for the fp32 kernel.  Lets a measurement name the kernel it timed. */
+                                   the bf16 kernels, 21..25 for the fp32 kernel.  Lets a measurement name the kernel it timed. */
 #define MS_QUERY_LAST_GRID 8     /* workgroups of the first of those launches: the compute units it ran on (at most the
                                    device's, less the reserved ones; fewer when that fills every round of the launch) */
 
@@ -341,8 +341,8 @@ int ms_probe_l2_lds_stream(const void *buffer, size_t buffer_bytes, int region_s
 
 /* Hook for tests and measurements (thread-local): later bf16 calls on this thread use tile variant `variant % 100`
  * (1..14, 0 = the library's choice) and split the contraction `variant / 100` ways (2..8, 0 = the library's choice;
- * a forced split needs a workspace and an output-stationary product).  21..24 name the fp32 kernel's tiles instead
- * (256x128, 128x192, 128x128, 64x64; split counts as above): fp32 calls then use that tile and bf16 calls the library's choice,
+ * a forced split needs a workspace and an output-stationary product).  21..25 name the fp32 kernel's tiles instead
+ * (256x128, 128x192, 128x128, 64x64, 192x192; split counts as above): fp32 calls then use that tile and bf16 calls the library's choice,
  * as fp32 calls do under 1..14.  Unknown ids are rejected with MS_ERR_ARG. */
 int ms_set_variant(int variant);
 

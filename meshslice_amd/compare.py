@@ -10,7 +10,7 @@
     dataflow (dimensions 512..16384, 0.02..3 TFLOP per product), S slices each.
 
 ``python3 -m meshslice_amd.compare fp32``
-    the fp32 kernel's default choice (tile and split count), each of its four tiles forced (ids 21..24, each with the
+    the fp32 kernel's default choice (tile and split count), each of its five tiles forced (ids 21..25, each with the
     split count the library would take for it) and the vendor library's product, output-stationary, on ten products
     from 512 x 512 x 1024 to 4096^3.
 
@@ -137,7 +137,7 @@ def chooser(cases, S, seed):
 
 FP32_SHAPES = [(4096, 4096, 4096), (8192, 2048, 2048), (3072, 3072, 4096), (2048, 3072, 4096), (2048, 6144, 2048), (2048, 2048, 8192),
                (1536, 1536, 4096), (1024, 2048, 4096), (1024, 1024, 1024), (512, 512, 1024)]
-FP32_TILES = (21, 22, 23, 24)      # 256x128, 128x192 (eight waves), 128x128, 64x64 (four waves)
+FP32_TILES = (21, 22, 23, 24, 25)      # 256x128, 128x192 (eight waves), 128x128, 64x64, 192x192 (four waves)
 
 
 def fp32(shapes=FP32_SHAPES):

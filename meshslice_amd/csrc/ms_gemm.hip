@@ -71,6 +71,7 @@ MS_INSTANTIATE_F32(4, 2, 2, 2)
 MS_INSTANTIATE_F32(4, 2, 1, 3)
 MS_INSTANTIATE_F32(2, 2, 2, 2)
 MS_INSTANTIATE_F32(2, 2, 1, 1)
+MS_INSTANTIATE_F32(2, 2, 3, 3)
 #undef MS_INSTANTIATE_F32
 
 namespace {
@@ -315,7 +316,7 @@ int launch_bf16_tile(const Problem &p, const DevFacts &dev, hipStream_t stream, 
 struct Pick { int v, splits; double cost; };
 
 constexpr int VARIANTS = 14;
-constexpr int F32_FIRST = 21, F32_LAST = 24;      // ids of the fp32 kernel's tiles (ms_set_variant, MS_QUERY_LAST_VARIANT)
+constexpr int F32_FIRST = 21, F32_LAST = 25;      // ids of the fp32 kernel's tiles (ms_set_variant, MS_QUERY_LAST_VARIANT)
 struct TileShape { int bm, bn; };
 constexpr TileShape TILE_OF[VARIANTS + 1] = {{0, 0},     {256, 256}, {256, 256}, {128, 128}, {256, 256}, {256, 192},
                                              {192, 256}, {256, 256}, {256, 192}, {192, 256}, {256, 384}, {384, 192},
@@ -475,8 +476,8 @@ int launch_bf16(const Problem &p, const DevFacts &dev, hipStream_t stream) {
   return launch_variant(single.v, single.splits, p, dev, stream);
 }
 
-// fp32 operands: gemm_f32_tile_kernel on one of its four tiles (ids F32_FIRST ..: 256 x 128 and 128 x 192 on eight
-// waves, 128 x 128 and 64 x 64 on four); `share`: two of the four-wave workgroups per compute unit
+// fp32 operands: gemm_f32_tile_kernel on one of its five tiles (ids F32_FIRST ..: 256 x 128 and 128 x 192 on eight
+// waves, 128 x 128, 64 x 64 and 192 x 192 on four); `share`: two workgroups of the 128 x 128 or 64 x 64 tile per compute unit
 int f32_split_refused(const Problem &p, const DevFacts &dev, int bm, int bn, int splits);
 
 template <int WGM, int WGN, int TM, int TN>
@@ -547,18 +548,21 @@ int f32_split_refused(const Problem &p, const DevFacts &dev, int bm, int bn, int
 // tile's, for a unit that holds one workgroup, and the factor by which a unit that holds two four-wave workgroups takes
 // longer over the pair.  Fitted to ten products from 512^2 x 1024 to 4096^3 (one round of 256 tiles of 128 x 192 on
 // 4096 contraction elements 363 us, of 256 x 128 468 us, of 128 x 128 on 8192 elements 510 us; 512 tiles of 64 x 64
-// shared 133 us, alone in two rounds 150 us; 1024 tiles of 128 x 128 shared 957 us).  Unlike the bf16 kernels this one
+// shared 133 us, alone in two rounds 150 us; 1024 tiles of 128 x 128 shared 957 us; one round of 256 tiles of 192 x 192,
+// four waves of 3 x 3 tiles each, 567 us).  Unlike the bf16 kernels this one
 // does not sit on the power limit: a partly filled round costs a whole one.
-struct F32Tile { int id, bm, bn; bool four_waves; double cost, shared; };
+struct F32Tile { int id, bm, bn; bool pairs; double cost, shared; };      // pairs: two such workgroups fit a compute unit
 constexpr F32Tile F32_TILES[] = {{F32_FIRST, 256, 128, false, 1.0, 0.0}, {F32_FIRST + 1, 128, 192, false, 1.0 / 0.967, 0.0},
-                                 {F32_FIRST + 2, 128, 128, true, 1.0 / 0.918, 1.88}, {F32_FIRST + 3, 64, 64, true, 1.0 / 0.78, 1.78}};
+                                 {F32_FIRST + 2, 128, 128, true, 1.0 / 0.918, 1.88}, {F32_FIRST + 3, 64, 64, true, 1.0 / 0.78, 1.78},
+                                 {F32_FIRST + 4, 192, 192, false, 1.0 / 0.93, 0.0}};
 
 int launch_f32_id(int id, bool share, int splits, const Problem &p, const DevFacts &dev, hipStream_t stream) {
   switch (id) {
     case F32_FIRST: return launch_f32_tile<4, 2, 2, 2>(p, dev, stream, id, false, splits);
     case F32_FIRST + 1: return launch_f32_tile<4, 2, 1, 3>(p, dev, stream, id, false, splits);
     case F32_FIRST + 2: return launch_f32_tile<2, 2, 2, 2>(p, dev, stream, id, share, splits);
-    default: return launch_f32_tile<2, 2, 1, 1>(p, dev, stream, id, share, splits);
+    case F32_FIRST + 3: return launch_f32_tile<2, 2, 1, 1>(p, dev, stream, id, share, splits);
+    default: return launch_f32_tile<2, 2, 3, 3>(p, dev, stream, id, false, splits);
   }
 }
 
@@ -589,7 +593,7 @@ int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
       const long items = tiles * splits;
       double cost = (double)((items + dev.cus - 1) / dev.cus) * area / splits;
       bool share = false;
-      if (t.four_waves && g_reserved_cus == 0 && items > dev.cus) {
+      if (t.pairs && g_reserved_cus == 0 && items > dev.cus) {
         const double both = (double)((items + 2L * dev.cus - 1) / (2L * dev.cus)) * area * t.shared / splits;
         if (both < cost) { cost = both; share = true; }
       }

@@ -187,10 +187,10 @@ def test_fp32_random_cases(flow):
         _run_and_compare(flow, ops, torch.float32, TOL_F32)
 
 
-@pytest.mark.parametrize("tile", [21, 22, 23, 24])
+@pytest.mark.parametrize("tile", [21, 22, 23, 24, 25])
 @pytest.mark.parametrize("flow", ["os", "ls", "rs"])
 def test_fp32_random_cases_on_every_tile(flow, tile):
-    """The fp32 kernel's four tiles (256x128 and 128x192 on eight waves, 128x128 and 64x64 on four), each forced."""
+    """The fp32 kernel's five tiles (256x128 and 128x192 on eight waves, 128x128, 64x64 and 192x192 on four), each forced."""
     lib = _lib.load()
     _lib.check(lib.ms_set_variant(tile))
     for idx, (m, n, k, S) in enumerate(SHAPES + [(200, 136, 100, 3), (300, 1000, 260, 1)]):
@@ -233,7 +233,7 @@ def test_bf16_output_is_one_rounding_of_the_fp32_accumulator():
     assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 3, 5, 8, 10, 11, 12, 13, 14, 21, 22, 23, 24])
+@pytest.mark.parametrize("variant", [0, 1, 3, 5, 8, 10, 11, 12, 13, 14, 21, 22, 23, 24, 25])
 @pytest.mark.parametrize("flow", ["ls", "rs"])
 @pytest.mark.parametrize("in_dtype", [torch.bfloat16, torch.float32])
 def test_bf16_chunks_are_one_rounding_of_the_fp32_chunks(flow, variant, in_dtype):
@@ -241,7 +241,7 @@ def test_bf16_chunks_are_one_rounding_of_the_fp32_chunks(flow, variant, in_dtype
     every chunk equals the round-to-nearest-even of the fp32 chunk of the same call, bit for bit, also on
     ragged shapes, and nothing is written outside a strided chunk."""
     if variant and (in_dtype == torch.float32) != (variant >= 21):
-        pytest.skip("variants 1-14 are tiles of the bf16 kernels, 21-24 of the fp32 kernel")
+        pytest.skip("variants 1-14 are tiles of the bf16 kernels, 21-25 of the fp32 kernel")
     _lib.check(_lib.load().ms_set_variant(variant))
     for (m, n, k, S) in [(512, 768, 256, 3), (264, 520, 72, 2), (1000, 776, 328, 2)]:
         ops = _rand_case(flow, m, n, k, S, seed=17 + variant, dtype=in_dtype)
@@ -387,7 +387,7 @@ def test_c_abi_rejects_bad_arguments():
     null, _k3 = _lib.ptr_array([0])
     assert call(pa=null) == _lib.MS_ERR_ARG
     assert lib.ms_set_variant(99) == _lib.MS_ERR_ARG
-    assert lib.ms_set_variant(25) == _lib.MS_ERR_ARG and lib.ms_set_variant(121) == _lib.MS_ERR_ARG      # fp32 tiles are 21-24; a split is 2..8 ways
+    assert lib.ms_set_variant(26) == _lib.MS_ERR_ARG and lib.ms_set_variant(121) == _lib.MS_ERR_ARG      # fp32 tiles are 21-25; a split is 2..8 ways
     with pytest.raises(ValueError):
         ms.gemm_os([a], [torch.zeros((32, 64), dtype=torch.bfloat16, device="cuda")])
     with pytest.raises(ValueError):

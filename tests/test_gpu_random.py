@@ -33,7 +33,7 @@ def test_random_cases(seed):
             flow = rnd.choice(["os", "ls", "rs"])
             dtype = rnd.choice([torch.bfloat16, torch.bfloat16, torch.float32])
             q = 8 if dtype == torch.bfloat16 else 4
-            variant = rnd.choice([0, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14]) if dtype == torch.bfloat16 else rnd.choice([0, 0, 21, 22, 23, 24])
+            variant = rnd.choice([0, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14]) if dtype == torch.bfloat16 else rnd.choice([0, 0, 21, 22, 23, 24, 25])
             top = 400 if rnd.random() < 0.15 else 120
             m, n, k = q * rnd.randint(1, top), 8 * rnd.randint(1, top), q * rnd.randint(1, 80)
             S = rnd.randint(1, 5)

@@ -30,10 +30,10 @@ def _slices(m, n, k, S, dtype, seed):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("variant", [0, 3, 7, 8, 9, 10, 11, 12, 13, 14, 208, 21, 22, 23, 24, 221, 322])
+@pytest.mark.parametrize("variant", [0, 3, 7, 8, 9, 10, 11, 12, 13, 14, 208, 21, 22, 23, 24, 25, 221, 322])
 def test_with_every_flag_set_the_gated_call_equals_the_plain_one(variant, dtype):
     if variant and (dtype == torch.float32) != (variant % 100 >= 21):
-        pytest.skip("variants 1-14 are tiles of the bf16 kernels, 21-24 of the fp32 kernel")
+        pytest.skip("variants 1-14 are tiles of the bf16 kernels, 21-25 of the fp32 kernel")
     S, m, n, k = 3, 520, 776, 136       # ragged tiles, a K tail in every slice
     A, B = _slices(m, n, k, S, dtype, seed=variant)
     lib = _lib.load()
