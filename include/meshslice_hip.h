@@ -125,8 +125,7 @@ int ms_gemm_os_ws(const void *const *A_slices, const void *const *B_slices, int 
  * split-contraction workspace is a fixed array inside the library's code object (4096 + 48 MiB per device, held until the
  * process ends); the call allocates and frees nothing.  A product whose exchange of partial tiles would not fit that
  * array is refused with MS_ERR_UNSUPPORTED (the message names the sizes) — use ms_gemm_os_ws there.  Only products that
- * split their contraction touch the array (few output tiles, a long contraction; bf16 operands only: an fp32 product
- * runs unsplit here); all such calls on one device share it.
+ * split their contraction touch the array (few output tiles, a long contraction); all such calls on one device share it.
  * Calls on one stream are ordered by the stream.  A call that arrives on another stream than the array's previous user
  * first waits for the device to go idle (hipDeviceSynchronize, under a per-device lock held until the call's kernels
  * are queued), so eager calls from several streams or host threads never meet in the array — at the price of that wait

@@ -575,12 +575,14 @@ int launch_f32_id(int id, bool share, int splits, const Problem &p, const DevFac
 constexpr double F32_SPLIT_FIX = 1.43e6, F32_SPLIT_PER_ELEMENT = 0.6;
 constexpr long F32_SPLIT_MIN_K = 256;      // contraction elements per split item, at least
 
-int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
+// the fp32 tile, whether its workgroups pair up on the units, and the split count with the lowest estimated cost (id 0: a
+// forced tile and split count that cannot be)
+struct F32Pick { int id, splits; bool share; };
+F32Pick pick_f32(const Problem &p, const DevFacts &dev) {
   const long chunks = p.flow == OS ? 1 : p.S;
   const long total_k = (long)p.K * (p.flow == OS ? p.S : 1);
   const bool forced_tile = g_variant >= F32_FIRST;
-  int best = 0, best_splits = 1;
-  bool best_share = false;
+  F32Pick best = {0, 1, false};
   double best_cost = 0.0;
   for (const F32Tile &t : F32_TILES) {
     if (forced_tile && g_variant != t.id) continue;
@@ -598,11 +600,16 @@ int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
         if (both < cost) { cost = both; share = true; }
       }
       if (splits > 1) cost += (F32_SPLIT_FIX + (double)splits * p.M * p.N * F32_SPLIT_PER_ELEMENT) / total_k;
-      if (best == 0 || cost < best_cost) { best = t.id; best_cost = cost; best_share = share; best_splits = splits; }
+      if (best.id == 0 || cost < best_cost) { best = {t.id, splits, share}; best_cost = cost; }
     }
   }
-  if (best == 0) return fail(MS_ERR_ARG, "contraction cannot be split %d ways on fp32 tile %d here", g_splits, g_variant);
-  return launch_f32_id(best, best_share, best_splits, p, dev, stream);
+  return best;
+}
+
+int launch_f32(const Problem &p, const DevFacts &dev, hipStream_t stream) {
+  const F32Pick best = pick_f32(p, dev);
+  if (best.id == 0) return fail(MS_ERR_ARG, "contraction cannot be split %d ways on fp32 tile %d here", g_splits, g_variant);
+  return launch_f32_id(best.id, best.share, best.splits, p, dev, stream);
 }
 
 // the device as this thread's launches may use it: without the compute units it has been told to leave free
@@ -837,23 +844,29 @@ MS_API int ms_gemm_os_noalloc(const void *const *A_slices, const void *const *B_
   Problem p = make_os(A_slices, B_slices, S, m, n, k_slice, lda, ldb, c1, ldc, in_dtype, out_dtype);
   int rc = validate(p);
   if (rc) return rc;
-  if (in_dtype != MS_DTYPE_BF16) return run(p, stream);     // without a workspace an fp32 product is never split: no scratch
   DevInfo *dev = nullptr;
   rc = dev_info(&dev);
   if (rc) return rc;
   // what the library would do with room to spare decides whether the built-in scratch is needed, and whether it is enough
   p.ws = reinterpret_cast<void *>(uintptr_t(256));    // stands for "a workspace": only its size is looked at here
   p.ws_bytes = ~size_t(0);
-  const Pick want = g_variant >= 1 && g_variant <= VARIANTS ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, usable(*dev));
-  if (want.splits <= 1) {
+  int splits = 1, bm = 0, bn = 0;
+  if (in_dtype == MS_DTYPE_BF16) {
+    const Pick want = g_variant >= 1 && g_variant <= VARIANTS ? Pick{g_variant, g_splits > 1 ? g_splits : 1, 0.0} : pick_variant(p, usable(*dev));
+    splits = want.splits; bm = TILE_OF[want.v].bm; bn = TILE_OF[want.v].bn;
+  } else {
+    const F32Pick want = pick_f32(p, usable(*dev));
+    splits = want.id ? want.splits : 1;
+    for (const F32Tile &t : F32_TILES) if (t.id == want.id) { bm = t.bm; bn = t.bn; }
+  }
+  if (splits <= 1) {
     // an unsplit product exchanges nothing (without a workspace the library makes the same choice: splits are only ever added)
     p.ws = nullptr;
     p.ws_bytes = 0;
     return run(p, stream);
   }
-  const TileShape t = TILE_OF[want.v];
-  const size_t tiles = (size_t)((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
-  const size_t need = WS_HEADER_BYTES + tiles * want.splits * t.bm * t.bn * sizeof(float);
+  const size_t tiles = (size_t)((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+  const size_t need = WS_HEADER_BYTES + tiles * splits * bm * bn * sizeof(float);
   if (need > NOALLOC_SCRATCH_BYTES)
     return fail(MS_ERR_UNSUPPORTED, "ms_gemm_os_noalloc: this product (m=%d n=%d k=%d x %d slices) would exchange %zu bytes of partial "
                 "tiles, the built-in scratch holds %zu; use ms_gemm_os_ws with a workspace of ms_workspace_bytes()",

@@ -1,6 +1,6 @@
 """The entry point that allocates nothing (``ms_gemm_os_noalloc``) through the C ABI: against ``ms_gemm_os_ws`` bit for
 bit on two calls in a row, the second with a smaller input, and against the float64 oracle (rel-Frobenius <= 1e-2,
-bf16 in / fp32 accumulate); the device's free memory does not move across the calls; calls that alternate between two
+bf16 in / fp32 accumulate; 1e-5 for the fp32 product); the device's free memory does not move across the calls; calls that alternate between two
 streams, and replays of a captured call, give the same bits; an over-sized product is refused with a message."""
 import ctypes
 
@@ -59,13 +59,33 @@ def test_no_alloc_entry_point_matches_the_workspace_entry_point():
     A3 = [_rand((4096, 512), 1.0, 41)]; B3 = [_rand((512, 4096), 0.02, 42)]
     got4, want4, splits4 = _both(L, A3, B3, 4096, 4096, 512, 1)
     assert splits4 == 1 and torch.equal(got4, want4)
-    # fp32 operands take the fp32 kernel (no scratch)
+    # fp32 operands take the fp32 kernel: a small product without the scratch ...
     a32 = torch.randn((256, 128), device="cuda"); b32 = torch.randn((128, 256), device="cuda")
     c32 = torch.empty((256, 256), device="cuda")
     pa, _ka = _lib.ptr_array([a32.data_ptr()]); pb, _kb = _lib.ptr_array([b32.data_ptr()])
     _lib.check(L.ms_gemm_os_noalloc(pa, pb, 1, 256, 256, 128, 128, 256, ctypes.c_void_p(c32.data_ptr()), 256,
                                     _lib.MS_DTYPE_F32, _lib.MS_DTYPE_F32, None))
+    assert L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == 1
     assert torch.allclose(c32, a32 @ b32, rtol=1e-4, atol=1e-3)
+    # ... and one that splits its contraction through it (1536 x 1536 x 4096 in two slices), the bits of ms_gemm_os_ws
+    g = torch.Generator(device="cuda").manual_seed(7)
+    A5 = [torch.randn((1536, 2048), generator=g, device="cuda") for _ in range(2)]
+    B5 = [torch.randn((2048, 1536), generator=g, device="cuda") * 0.02 for _ in range(2)]
+    pa, _ka = _lib.ptr_array([t.data_ptr() for t in A5]); pb, _kb = _lib.ptr_array([t.data_ptr() for t in B5])
+    ws = local_gemm.workspace("cuda")
+    want5 = torch.empty((1536, 1536), device="cuda"); got5 = torch.zeros((1536, 1536), device="cuda")
+    head5 = lambda C: (pa, pb, 2, 1536, 1536, 2048, 2048, 1536, ctypes.c_void_p(C.data_ptr()), 1536, _lib.MS_DTYPE_F32, _lib.MS_DTYPE_F32)
+    _lib.check(L.ms_gemm_os_ws(*head5(want5), _lib.MS_ACT_NONE, None, 0, None, None, ctypes.c_void_p(ws.data_ptr()), ws.numel(), None))
+    splits5, tile5 = L.ms_query(_lib.MS_QUERY_LAST_SPLITS), L.ms_query(_lib.MS_QUERY_LAST_VARIANT)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    _lib.check(L.ms_gemm_os_noalloc(*head5(got5), None))
+    assert splits5 > 1 and L.ms_query(_lib.MS_QUERY_LAST_SPLITS) == splits5 and L.ms_query(_lib.MS_QUERY_LAST_VARIANT) == tile5
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.equal(got5, want5)
+    ref5 = sum(a[:48].double() @ b.double() for a, b in zip(A5, B5))
+    assert ((got5[:48].double() - ref5).norm() / ref5.norm()).item() <= 1e-5
 
 
 def _noalloc(L, A, B, C, stream):
